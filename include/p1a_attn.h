@@ -1,0 +1,132 @@
+/*
+ * p1a_attn.h - C ABI of the MI355X (gfx950) paged-KV attention library: quantize-on-append KV write, split-K
+ * decode / MTP multi-token verify, chunked causal prefill and the fused sigmoid output gate.
+ *
+ * Each entry point replaces one function of the reference engine's C++ attention surface (namespace p100e::fast);
+ * the reference file:line is given with every declaration (paths relative to the reference tree). The C++ mirror of
+ * that surface, with the reference's names and argument order, is include/p100e_fast_attn.hpp; it only calls the
+ * functions below.
+ *
+ * Conventions shared by all entry points
+ *   - All tensor pointers are DEVICE pointers; `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *   - Return value: 0 = work enqueued; negative (P1A_E_*) = refused, NOTHING was launched and the outputs are
+ *     untouched; a diagnostic goes to stderr and to p1a_last_error(). No exceptions, no host synchronisation.
+ *   - Positions (`p0_dev`, `pos_rows`) and page tables (`pt`, `rtab`) are read ON THE DEVICE when the kernels run,
+ *     so a captured hipGraph replays correctly at any depth.
+ *   - Split-K scratch is owned by the library per (device, stream) and is allocated on the first call; call
+ *     p1a_warmup() (or one eager call at the largest row count) before hipGraph capture so the pointer never changes.
+ */
+#ifndef P1A_ATTN_H
+#define P1A_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* KV storage modes; values equal the reference's (= the ggml type ids). src/fast/attn.cuh:14-16 */
+#define P1A_KV_F16  1u
+#define P1A_KV_Q4_0 2u
+#define P1A_KV_Q8_0 8u
+
+#define P1A_OK            0
+#define P1A_E_SHAPE      (-1) /* unsupported shape / type / alignment */
+#define P1A_E_ARG        (-2) /* null or inconsistent argument */
+#define P1A_E_SCRATCH    (-3) /* scratch allocation failed or caller scratch too small */
+#define P1A_E_LAUNCH     (-4) /* the HIP runtime reported a launch error */
+
+#define P1A_MAX_ROWS 32 /* query rows per p1a_attn_decode call (the reference allows 8: src/fast/attn.cuh:66) */
+
+/*
+ * POD copy of the reference's `struct kv_cache` (src/fast/attn.cuh:18-32); same fields, same meaning.
+ * Position p of query row t lives at
+ *     base + pt[(rtab ? rtab[t] : 0) + (p >> psh)] * pstride + (p & (2^psh - 1)) * row_bytes      (pt != NULL)
+ *     base + p * row_bytes                                                                        (pt == NULL)
+ * with base = k or v. Row layouts (per position: Hkv heads back to back):
+ *     f16  : D halves per head
+ *     q8_0 : per head D/32 f16 scales, then D int8 codes (272 B at D = 256)            src/fast/kv_q8.cuh:1-5
+ *     q4_0 : per head D/32 ggml block_q4_0 (f16 d, 16 B: byte i = v[i] | v[i+16] << 4)   src/fast/attn.cuh:4-5
+ * The layer is selected by the k / v base pointers, the slot by pt (or rtab[t]), the storage mode by type.
+ */
+typedef struct p1a_kv {
+    uint32_t type;
+    int32_t n_ctx, Hkv, D;
+    void *k;
+    void *v;
+    const int32_t *pt;
+    const int32_t *rtab;
+    int32_t psh;
+    size_t pstride;
+} p1a_kv;
+
+/* bytes of one position (all kv heads) of K or V. Replaces kv_row_bytes, src/fast/attn.cu:501-503. */
+size_t p1a_kv_row_bytes(uint32_t type, int Hkv, int D);
+
+/*
+ * Quantize-on-append KV write: k, v [T][Hkv][D] f32 -> cache rows. Row t goes to position
+ *     pos_rows[t]            when pos_rows != NULL (each row in its own sequence, table pt + rtab[t])
+ *     *p0_dev + t            else when p0_dev != NULL
+ *     p0 + t                 otherwise.
+ * Codes and scales are bit-identical to ggml's quantize_row_q8_0_ref / quantize_row_q4_0_ref.
+ * Replaces kv_append (src/fast/attn.cuh:37-38, attn.cu:583-585), kv_append_dev (attn.cuh:58, attn.cu:587-589) and
+ * the cache-write half of attn_prep in its device-position mode (src/fast/fused.cuh:101-113, fused.cu:512-526,563-572).
+ * k, v must be 16-byte aligned; D % 32 == 0 for the quantized types.
+ */
+int p1a_kv_append(const p1a_kv *c, const float *k, const float *v, int p0, const int32_t *p0_dev,
+                  const int32_t *pos_rows, int T, void *stream);
+
+/*
+ * Decode / MTP-verify attention: q, out [T][Hq][D] f32;
+ *     out[t][h] = softmax_{j <= pos(t)} (scale * q[t][h] . K[j][h / (Hq/Hkv)]) . V[j][h / (Hq/Hkv)]
+ * and, when gate != NULL (gate [T][Hq*D] f32), out *= 1 / (1 + exp(-gate)) fused into the final merge.
+ * pos(t) = pos_rows[t] | *p0_dev + t | p0 + t as for p1a_kv_append. With pos_rows, `rows_per_seq` consecutive rows
+ * share one sequence (the page table of the first row of each group): 1 = every row on its own (the reference's
+ * attn_decode_rows), n > 1 = n-token verify blocks of several sequences in one call, each block reading its KV once.
+ * Without pos_rows all T rows belong to one sequence and share the KV read in groups of up to 4 rows.
+ * The key partition does not depend on T, p0 or the batch composition: row t of any call is bitwise the T = 1 call
+ * at pos(t) on that sequence, and a paged cache gives the bits of the contiguous one.
+ * Replaces attn_decode (src/fast/attn.cuh:44, attn.cu:638-648), attn_decode_dev (attn.cuh:59-60, attn.cu:656-666),
+ * attn_decode_rows (attn.cuh:64-65, attn.cu:650-654) and attn_decode2 (src/fast/attn_dec2.cuh:17-18); the gate
+ * replaces the separate sigmoid_mul launch (src/kernels.cu:85-93).
+ */
+int p1a_attn_decode(const float *q, const p1a_kv *c, float *out, const float *gate, int T, int p0,
+                    const int32_t *p0_dev, const int32_t *pos_rows, int rows_per_seq, int Hq, float scale,
+                    void *stream);
+
+/*
+ * Chunked causal prefill: q, out [T][Hq][D] f32, query t at position p0 + t sees cache positions 0..p0+t of ONE
+ * sequence (page table pt + (rtab ? rtab[0] : 0)); the cache must already hold positions 0..p0+T-1 (append first).
+ * fp16 MFMA products with fp32 accumulation; gate as in p1a_attn_decode. `scratch` is caller-supplied device memory
+ * of at least p1a_attn_prefill_scratch_bytes(...) bytes (may be NULL when that is 0).
+ * Replaces attn_prefill (src/fast/attn.cuh:46-50) and attn_fold (src/fast/attn_fold.cuh:19-26).
+ */
+int p1a_attn_prefill(const float *q, const p1a_kv *c, float *out, const float *gate, int T, int p0, int Hq,
+                     float scale, void *scratch, size_t scratch_bytes, void *stream);
+/* Replaces attn_fold_scratch_bytes (src/fast/attn_fold.cuh:19). */
+size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D);
+
+/* Standalone sigmoid gate x[i] *= 1 / (1 + exp(-g[i])). Replaces k::sigmoid_mul, src/kernels.cu:85-93. */
+int p1a_sigmoid_mul(float *x, const float *g, size_t n, void *stream);
+
+/*
+ * Allocate the split-K scratch of (current device, stream) for up to `rows` query rows of Hq heads of size D, so that
+ * later calls on that stream never allocate (graph capture). Mirrors the warm-up call the reference asks for
+ * (src/fast/attn.cuh:40-42).
+ */
+int p1a_warmup(int rows, int Hq, int Hkv, int D, void *stream);
+/* split-stream count used for Hkv kv heads on the current device / override it (0 = default). Mirror
+ * attn_dec2_nsplit / attn_dec2_set_nsplit, src/fast/attn_dec2.cuh:19-20. Never change it between graph captures. */
+int p1a_get_nsplit(int Hkv);
+void p1a_set_nsplit(int n);
+/* free every scratch buffer of the current process (after synchronising the devices that own them) */
+void p1a_release(void);
+
+const char *p1a_last_error(void);
+const char *p1a_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* P1A_ATTN_H */

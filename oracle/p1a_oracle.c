@@ -1,0 +1,312 @@
+/* CPU oracle (TEST INFRASTRUCTURE) - see p1a_oracle.h for scope and for what pins each function. */
+#include "p1a_oracle.h"
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ---- f16 <-> f32, IEEE round-to-nearest-even, subnormals kept (the device uses v_cvt_f16_f32 in RNE mode;
+ * the reference uses __float2half, src/fast/kv_q8.cuh:25,48) ---- */
+uint16_t orc_f32_to_f16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const uint32_t a = x & 0x7fffffffu;
+    if (a >= 0x7f800000u) return (uint16_t) (sign | 0x7c00u | (a > 0x7f800000u ? 0x200u | ((a >> 13) & 0x3ffu) : 0u));
+    if (a >= 0x477ff000u) return (uint16_t) (sign | 0x7c00u);           /* rounds to >= 65520 -> inf */
+    if (a >= 0x38800000u) {                                           /* normal half */
+        const uint32_t m = a - 0x38000000u;                           /* rebias exponent 127 -> 15 */
+        const uint32_t r = m + 0xfffu + ((m >> 13) & 1u);             /* RNE on the 13 dropped bits */
+        return (uint16_t) (sign | (r >> 13));
+    }
+    if (a < 0x33000000u) return (uint16_t) sign;                      /* < 2^-25 -> 0 (ties at 2^-25 go to even = 0) */
+    {                                                                 /* subnormal half */
+        const int e = (int) (a >> 23);                                /* 102..112 */
+        const uint32_t m = (a & 0x7fffffu) | 0x800000u;               /* 24-bit significand */
+        const int sh = 126 - e;                                       /* 14..24 bits dropped */
+        const uint32_t q = m >> sh, rem = m & ((1u << sh) - 1u), half = 1u << (sh - 1);
+        uint32_t r = q;
+        if (rem > half || (rem == half && (q & 1u))) ++r;
+        return (uint16_t) (sign | r);
+    }
+}
+
+float orc_f16_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t) (h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1fu, m = h & 0x3ffu;
+    uint32_t x;
+    if (e == 0x1f) x = sign | 0x7f800000u | (m << 13);
+    else if (e) x = sign | ((e + 112u) << 23) | (m << 13);
+    else if (!m) x = sign;
+    else {
+        int s = 0;
+        uint32_t mm = m;
+        while (!(mm & 0x400u)) { mm <<= 1; ++s; }
+        x = sign | ((uint32_t) (113 - s) << 23) | ((mm & 0x3ffu) << 13);
+    }
+    float f;
+    memcpy(&f, &x, 4);
+    return f;
+}
+
+/* src/fast/attn.cu:501-503 */
+size_t orc_kv_row_bytes(uint32_t type, int Hkv, int D) {
+    if (type == ORC_KV_F16) return (size_t) Hkv * D * 2;
+    if (type == ORC_KV_Q8_0) return (size_t) Hkv * (D / 32) * 34;
+    return (size_t) Hkv * (D / 32) * 18;
+}
+
+/* src/fast/kv_page.cuh:21-31, src/fast/attn.cuh:23-27 */
+size_t orc_kv_off(const orc_kv *c, int t, int p) {
+    const size_t rowb = orc_kv_row_bytes(c->type, c->Hkv, c->D);
+    if (!c->pt) return (size_t) p * rowb;
+    const int32_t *tab = c->rtab ? c->pt + c->rtab[t] : c->pt;
+    return (size_t) tab[p >> c->psh] * c->pstride + (size_t) (p & ((1 << c->psh) - 1)) * rowb;
+}
+
+/* src/fast/kv_q8.cuh:20-26 (= ggml quantize_row_q8_0_ref, ggml-quants.c:276-299):
+ * d = amax / 127 (f32), id = d ? 1/d : 0, q = roundf(x * id) (half away from zero), scale stored as RNE f16 of d. */
+void orc_quant_q8_0_block(const float *x, uint16_t *d_bits, int8_t *q) {
+    float amax = 0.0f;
+    for (int j = 0; j < 32; ++j) {
+        const float a = fabsf(x[j]);
+        if (a > amax) amax = a;
+    }
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    *d_bits = orc_f32_to_f16(d);
+    for (int j = 0; j < 32; ++j) {
+        volatile float p = x[j] * id; /* product rounded to f32 before roundf */
+        q[j] = (int8_t) (int) roundf(p);
+    }
+}
+
+/* src/fast/kv_q8.cuh:32-49 (= ggml quantize_row_q4_0_ref, ggml-quants.c:113-147): max = the signed value of largest
+ * magnitude (first one on ties; 0 when every |x| is 0), d = max / -8, q = min(15, (int)(x * id + 8.5f)) with the
+ * product and the sum rounded separately; byte j = q[j] | q[j + 16] << 4. */
+void orc_quant_q4_0_block(const float *x, uint8_t *blk18) {
+    float amax = 0.0f, mx = 0.0f;
+    for (int j = 0; j < 32; ++j) {
+        const float a = fabsf(x[j]);
+        if (amax < a) { amax = a; mx = x[j]; }
+    }
+    const float d = mx / -8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const uint16_t db = orc_f32_to_f16(d);
+    blk18[0] = (uint8_t) (db & 0xff);
+    blk18[1] = (uint8_t) (db >> 8);
+    for (int j = 0; j < 16; ++j) {
+        volatile float p0 = x[j] * id, p1 = x[j + 16] * id;
+        volatile float s0 = p0 + 8.5f, s1 = p1 + 8.5f;
+        int q0 = (int) s0, q1 = (int) s1;
+        if (q0 > 15) q0 = 15;
+        if (q1 > 15) q1 = 15;
+        blk18[2 + j] = (uint8_t) (q0 | (q1 << 4));
+    }
+}
+
+/* row layouts: src/fast/attn.cuh:1-7 and src/fast/kv_q8.cuh:1-5 (q8_0: per head D/32 f16 scales then D int8;
+ * q4_0: D/32 ggml blocks of 18 B; f16: plain halves); appends: src/fast/attn.cu:245-283 */
+static void append_head(uint32_t type, int D, const float *x, uint8_t *dst) {
+    if (type == ORC_KV_F16) {
+        for (int i = 0; i < D; ++i) {
+            const uint16_t h = orc_f32_to_f16(x[i]);
+            dst[2 * i] = (uint8_t) (h & 0xff);
+            dst[2 * i + 1] = (uint8_t) (h >> 8);
+        }
+    } else if (type == ORC_KV_Q8_0) {
+        const int nb = D / 32;
+        for (int b = 0; b < nb; ++b) {
+            uint16_t d;
+            orc_quant_q8_0_block(x + 32 * b, &d, (int8_t *) dst + 2 * nb + 32 * b);
+            dst[2 * b] = (uint8_t) (d & 0xff);
+            dst[2 * b + 1] = (uint8_t) (d >> 8);
+        }
+    } else {
+        for (int b = 0; b < D / 32; ++b) orc_quant_q4_0_block(x + 32 * b, dst + 18 * b);
+    }
+}
+
+static size_t head_bytes(uint32_t type, int D) { return orc_kv_row_bytes(type, 1, D); }
+
+void orc_kv_append_rows(const orc_kv *c, const float *k, const float *v, const int32_t *pos, int T) {
+    const size_t hb = head_bytes(c->type, c->D);
+    for (int t = 0; t < T; ++t) {
+        const size_t o = orc_kv_off(c, t, pos[t]);
+        for (int h = 0; h < c->Hkv; ++h) {
+            const size_t src = ((size_t) t * c->Hkv + h) * c->D;
+            append_head(c->type, c->D, k + src, (uint8_t *) c->k + o + h * hb);
+            append_head(c->type, c->D, v + src, (uint8_t *) c->v + o + h * hb);
+        }
+    }
+}
+
+/* element reader: tests/fast_attn_test.cu:34-44 (value = code * f32(f16 scale); q4_0 value = (nibble - 8) * scale) */
+void orc_kv_read_head(const orc_kv *c, int which, int t, int p, int hk, float *dst) {
+    const uint8_t *row = (const uint8_t *) (which ? c->v : c->k) + orc_kv_off(c, t, p) + hk * head_bytes(c->type, c->D);
+    const int D = c->D;
+    if (c->type == ORC_KV_F16) {
+        for (int i = 0; i < D; ++i) dst[i] = orc_f16_to_f32((uint16_t) (row[2 * i] | (row[2 * i + 1] << 8)));
+    } else if (c->type == ORC_KV_Q8_0) {
+        const int nb = D / 32;
+        const int8_t *qs = (const int8_t *) row + 2 * nb;
+        for (int b = 0; b < nb; ++b) {
+            const float d = orc_f16_to_f32((uint16_t) (row[2 * b] | (row[2 * b + 1] << 8)));
+            for (int i = 0; i < 32; ++i) dst[32 * b + i] = d * (float) qs[32 * b + i];
+        }
+    } else {
+        for (int b = 0; b < D / 32; ++b) {
+            const uint8_t *blk = row + 18 * b;
+            const float d = orc_f16_to_f32((uint16_t) (blk[0] | (blk[1] << 8)));
+            for (int i = 0; i < 16; ++i) {
+                dst[32 * b + i] = (float) ((int) (blk[2 + i] & 15) - 8) * d;
+                dst[32 * b + 16 + i] = (float) ((int) (blk[2 + i] >> 4) - 8) * d;
+            }
+        }
+    }
+}
+
+/* src/kernels.cu:85-88 */
+void orc_gate(float *x, const float *g, size_t n) {
+    for (size_t i = 0; i < n; ++i) x[i] *= 1.0f / (1.0f + expf(-g[i]));
+}
+
+/* src/kernels.cu:34-42 with w == NULL */
+void orc_rmsnorm_heads(float *x, size_t nheads, int D, float eps) {
+    for (size_t r = 0; r < nheads; ++r) {
+        float *xr = x + r * D;
+        float ss = 0.0f;
+        for (int i = 0; i < D; ++i) ss += xr[i] * xr[i];
+        const float sc = 1.0f / sqrtf(ss / (float) D + eps);
+        for (int i = 0; i < D; ++i) xr[i] = xr[i] * sc;
+    }
+}
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/*
+ * Attention of src/kernels.cu:143-166 (attention_k): for query row t and head h, kv head hk = h / (Hq / Hkv),
+ * n_kv = pos[t] + 1 visible keys, score_j = (q . k_j) * scale, mx = max score, den = sum exp(score - mx),
+ * out = sum exp(score_j - mx) v_j / den, all fp32; then the gate of src/kernels.cu:85-88 when given.
+ * Keys are walked in fixed chunks of ORC_CHUNK so that the partial sums (and hence the bits) do not depend on the
+ * thread count; the reference kernel sums sequentially, the difference is a few fp32 ulps.
+ * The cache is read through the page table (src/fast/kv_page.cuh:21-31) and dequantized as tests/fast_attn_test.cu:34-44.
+ */
+#define ORC_CHUNK 256
+
+int orc_attn_rows(const orc_kv *c, const float *q, float *out, const float *gate, int T, const int32_t *pos, int Hq,
+                  float scale, int f64) {
+    const int D = c->D, Hkv = c->Hkv;
+    if (Hkv <= 0 || Hq % Hkv || D <= 0 || T < 0) return -1;
+    const int G = Hq / Hkv;
+    for (int t = 0; t < T; ++t) {
+        for (int hk = 0; hk < Hkv; ++hk) {
+            const int n = pos[t] + 1;
+            const int nch = (n + ORC_CHUNK - 1) / ORC_CHUNK;
+            float *sc = (float *) malloc((size_t) G * n * sizeof(float));
+            double *scd = f64 ? (double *) malloc((size_t) G * n * sizeof(double)) : NULL;
+            double *part = (double *) calloc((size_t) nch * G * D, sizeof(double));
+            if (!sc || !part || (f64 && !scd)) { free(sc); free(scd); free(part); return -2; }
+            /* pass 1: scores */
+#pragma omp parallel
+            {
+                float *row = (float *) malloc((size_t) D * sizeof(float));
+#pragma omp for schedule(static)
+                for (int j = 0; j < n; ++j) {
+                    orc_kv_read_head(c, 0, t, j, hk, row);
+                    for (int g = 0; g < G; ++g) {
+                        const float *qr = q + ((size_t) t * Hq + hk * G + g) * D;
+                        if (f64) {
+                            double d = 0.0;
+                            for (int i = 0; i < D; ++i) d += (double) qr[i] * (double) row[i];
+                            scd[(size_t) g * n + j] = d * (double) scale;
+                        } else {
+                            float d8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                            for (int i = 0; i < D; i += 8)
+                                for (int u = 0; u < 8; ++u) d8[u] += qr[i + u] * row[i + u];
+                            const float d = ((d8[0] + d8[4]) + (d8[2] + d8[6])) + ((d8[1] + d8[5]) + (d8[3] + d8[7]));
+                            sc[(size_t) g * n + j] = d * scale;
+                        }
+                    }
+                }
+                free(row);
+            }
+            /* max and denominator per head */
+            double mxd[64], dend[64];
+            float mxf[64], denf[64];
+            if (G > 64) { free(sc); free(scd); free(part); return -1; }
+            for (int g = 0; g < G; ++g) {
+                if (f64) {
+                    double mx = -INFINITY, den = 0.0;
+                    for (int j = 0; j < n; ++j) mx = scd[(size_t) g * n + j] > mx ? scd[(size_t) g * n + j] : mx;
+                    for (int j = 0; j < n; ++j) den += exp(scd[(size_t) g * n + j] - mx);
+                    mxd[g] = mx; dend[g] = den;
+                } else {
+                    float mx = -INFINITY, den = 0.0f;
+                    for (int j = 0; j < n; ++j) mx = fmaxf(mx, sc[(size_t) g * n + j]);
+                    for (int j = 0; j < n; ++j) den += expf(sc[(size_t) g * n + j] - mx);
+                    mxf[g] = mx; denf[g] = den;
+                }
+            }
+            /* pass 2: weighted V, per fixed chunk */
+#pragma omp parallel
+            {
+                float *row = (float *) malloc((size_t) D * sizeof(float));
+                float *accf = (float *) malloc((size_t) G * D * sizeof(float));
+#pragma omp for schedule(static)
+                for (int ch = 0; ch < nch; ++ch) {
+                    const int j0 = ch * ORC_CHUNK, j1 = j0 + ORC_CHUNK < n ? j0 + ORC_CHUNK : n;
+                    double *pa = part + (size_t) ch * G * D;
+                    memset(accf, 0, (size_t) G * D * sizeof(float));
+                    for (int j = j0; j < j1; ++j) {
+                        orc_kv_read_head(c, 1, t, j, hk, row);
+                        for (int g = 0; g < G; ++g) {
+                            if (f64) {
+                                const double p = exp(scd[(size_t) g * n + j] - mxd[g]);
+                                for (int i = 0; i < D; ++i) pa[(size_t) g * D + i] += p * (double) row[i];
+                            } else {
+                                const float p = expf(sc[(size_t) g * n + j] - mxf[g]);
+                                float *a = accf + (size_t) g * D;
+                                for (int i = 0; i < D; ++i) a[i] += p * row[i];
+                            }
+                        }
+                    }
+                    if (!f64) for (int i = 0; i < G * D; ++i) pa[i] = (double) accf[i];
+                }
+                free(row);
+                free(accf);
+            }
+            for (int g = 0; g < G; ++g) {
+                float *o = out + ((size_t) t * Hq + hk * G + g) * D;
+                for (int i = 0; i < D; ++i) {
+                    if (f64) {
+                        double a = 0.0;
+                        for (int ch = 0; ch < nch; ++ch) a += part[((size_t) ch * G + g) * D + i];
+                        o[i] = (float) (a / dend[g]);
+                    } else {
+                        float a = 0.0f;
+                        for (int ch = 0; ch < nch; ++ch) a += (float) part[((size_t) ch * G + g) * D + i];
+                        o[i] = a / denf[g];
+                    }
+                }
+            }
+            free(sc); free(scd); free(part);
+        }
+    }
+    if (gate) {
+        if (f64) {
+            for (size_t i = 0; i < (size_t) T * Hq * D; ++i) out[i] = (float) ((double) out[i] / (1.0 + exp(-(double) gate[i])));
+        } else {
+            orc_gate(out, gate, (size_t) T * Hq * D);
+        }
+    }
+    return 0;
+}

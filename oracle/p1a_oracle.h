@@ -1,0 +1,69 @@
+/*
+ * CPU oracle for the paged-KV attention path (TEST INFRASTRUCTURE, not product code).
+ *
+ * Only tests, the smoke check and the benchmark's cpu_baseline leg may link or call this. It is a plain-C
+ * restatement of the arithmetic of the reference engine's attention path; every function cites the reference
+ * file:line it follows (paths relative to the reference tree).
+ *
+ * How each function is pinned (see tests/test_oracle_*.py):
+ *   orc_quant_q8_0_block / orc_quant_q4_0_block : golden vectors produced by the reference's vendored ggml C
+ *       quantizers (tests/golden/quant_golden.npz) + closed forms (zero block, +-amax codes, ties, half-way cases).
+ *   orc_f32_to_f16 / orc_f16_to_f32           : exhaustive against numpy float16 (all 65536 halves; 2^20 floats).
+ *   orc_kv_off / orc_kv_row_bytes / row layout : byte formulas of src/fast/attn.cuh:1-32 and the independent
+ *       element reader of tests/fast_attn_test.cu:34-44, restated in numpy; paged(perm) == contiguous invariant.
+ *   orc_attn_rows                              : numpy float64 softmax(QK^T)V on the dequantized cache, n = 1,
+ *       equal-V, dominant-logit, causality and shift-invariance closed forms.
+ *   orc_gate                                   : g = 0 -> x0.5, sigma(g) + sigma(-g) = 1.
+ * No function of this file is "parity unpinned".
+ */
+#ifndef P1A_ORACLE_H
+#define P1A_ORACLE_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { ORC_KV_F16 = 1, ORC_KV_Q4_0 = 2, ORC_KV_Q8_0 = 8 }; /* src/fast/attn.cuh:14-16 */
+
+/* host-memory twin of the engine's kv_cache descriptor (src/fast/attn.cuh:18-32) */
+typedef struct orc_kv {
+    uint32_t type;
+    int32_t n_ctx, Hkv, D;
+    void *k, *v;
+    const int32_t *pt;   /* page table(s); NULL = contiguous */
+    const int32_t *rtab; /* per-row element offsets into pt; NULL = 0 */
+    int32_t psh;
+    size_t pstride;
+} orc_kv;
+
+uint16_t orc_f32_to_f16(float f);
+float orc_f16_to_f32(uint16_t h);
+
+size_t orc_kv_row_bytes(uint32_t type, int Hkv, int D);
+/* byte offset of position p of query row t inside the K (or V) region */
+size_t orc_kv_off(const orc_kv *c, int t, int p);
+
+/* one 32-value block: scale bits (f16) + 32 int8 codes */
+void orc_quant_q8_0_block(const float *x, uint16_t *d_bits, int8_t *q);
+/* one 32-value block -> the 18-byte ggml block_q4_0 */
+void orc_quant_q4_0_block(const float *x, uint8_t *blk18);
+
+/* k, v: [T][Hkv][D] f32 -> cache rows at pos[t] (t-th row uses rtab[t] when present) */
+void orc_kv_append_rows(const orc_kv *c, const float *k, const float *v, const int32_t *pos, int T);
+/* dequantize one (position, kv head) row of K (which = 0) or V (which = 1) into dst[D] */
+void orc_kv_read_head(const orc_kv *c, int which, int t, int p, int hk, float *dst);
+
+/* q, out: [T][Hq][D] f32. Row t sees positions 0..pos[t] of its own sequence. gate ([T][Hq*D], may be NULL)
+ * multiplies the normalised output by sigmoid(gate). f64 != 0: all arithmetic in double (error budgeting). */
+int orc_attn_rows(const orc_kv *c, const float *q, float *out, const float *gate, int T, const int32_t *pos, int Hq,
+                  float scale, int f64);
+void orc_gate(float *x, const float *g, size_t n);
+/* per-head RMS norm with unit weight, in place: x * rsqrt(mean(x^2) + eps) */
+void orc_rmsnorm_heads(float *x, size_t nheads, int D, float eps);
+int orc_num_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,194 @@
+// extern "C" layer of the paged-KV attention library: argument validation (refusals launch nothing), split-K
+// scratch ownership per (device, stream), split-count bookkeeping. All device work lives in the other .hip files.
+#include "p1a_common.hpp"
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+namespace p1a {
+
+static thread_local char g_err[256] = "";
+
+void set_error(const char * fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    fprintf(stderr, "p1a_attn: %s\n", g_err);
+}
+
+namespace {
+
+// Split partials per (device, stream): calls on different streams of one device may overlap; a stream keeps its
+// buffer (captured graphs hold the pointer), which only ever grows, and only outside capture.
+struct scratch { int dev = -1; hipStream_t s = nullptr; float * o = nullptr; float * ml = nullptr; size_t cap_o = 0, cap_ml = 0; };
+constexpr int MAX_SCR = 64;
+scratch g_scr[MAX_SCR];
+int g_nscr = 0;
+std::mutex g_mu;
+int g_nsplit_override = 0;
+int g_cus[16] = {0};
+
+int cu_count() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    int & n = g_cus[dev & 15];
+    if (!n && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256;
+    return n;
+}
+
+scratch * scratch_for(hipStream_t s, size_t need_o, size_t need_ml) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lk(g_mu);
+    scratch * e = nullptr;
+    for (int i = 0; i < g_nscr; ++i) if (g_scr[i].dev == dev && g_scr[i].s == s) e = &g_scr[i];
+    if (!e) {
+        if (g_nscr == MAX_SCR) { set_error("too many (device, stream) pairs"); return nullptr; }
+        e = &g_scr[g_nscr++];
+        e->dev = dev; e->s = s;
+    }
+    if (need_o > e->cap_o || need_ml > e->cap_ml) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
+            set_error("split scratch would have to grow during stream capture: call p1a_warmup first");
+            return nullptr;
+        }
+        float * no = nullptr, * nm = nullptr;
+        if (hipMalloc(&no, need_o) != hipSuccess || hipMalloc(&nm, need_ml) != hipSuccess) {
+            (void) hipGetLastError();
+            if (no) (void) hipFree(no);
+            set_error("split scratch allocation failed (%zu bytes)", need_o + need_ml);
+            return nullptr;
+        }
+        if (e->o) { (void) hipStreamSynchronize(s); (void) hipFree(e->o); (void) hipFree(e->ml); }
+        e->o = no; e->ml = nm; e->cap_o = need_o; e->cap_ml = need_ml;
+    }
+    return e;
+}
+
+bool kv_ok(const p1a_kv * c, const char * who) {
+    if (!c || !c->k || !c->v) { set_error("%s: null cache", who); return false; }
+    if (c->type != P1A_KV_F16 && c->type != P1A_KV_Q8_0 && c->type != P1A_KV_Q4_0) { set_error("%s: unknown KV type %u", who, c->type); return false; }
+    if (c->Hkv < 1 || c->D < 32 || c->D % 32 || c->D > 512) { set_error("%s: unsupported shape (Hkv=%d D=%d)", who, c->Hkv, c->D); return false; }
+    if (c->pt && (c->psh < 0 || c->psh > 24 || c->pstride == 0)) { set_error("%s: bad page geometry (psh=%d pstride=%zu)", who, c->psh, c->pstride); return false; }
+    return true;
+}
+
+int nsplit_for(const p1a_kv & c, int Hq) {
+    static const int env = getenv("P1A_DEC_SPLIT") ? atoi(getenv("P1A_DEC_SPLIT")) : 0;
+    if (g_nsplit_override > 0) return g_nsplit_override;
+    if (env > 0) return env;
+    return decode_default_nsplit(c, Hq, cu_count());
+}
+
+}   // namespace
+}   // namespace p1a
+
+using namespace p1a;
+
+extern "C" {
+
+size_t p1a_kv_row_bytes(uint32_t type, int Hkv, int D) {
+    return type == P1A_KV_F16 ? (size_t) Hkv * D * 2 : type == P1A_KV_Q8_0 ? (size_t) Hkv * (D / 32) * 34 : (size_t) Hkv * (D / 32) * 18;
+}
+
+int p1a_kv_append(const p1a_kv * c, const float * k, const float * v, int p0, const int32_t * p0_dev,
+                  const int32_t * pos_rows, int T, void * stream) {
+    if (!kv_ok(c, "p1a_kv_append")) return P1A_E_ARG;
+    if (!k || !v || T < 0) { set_error("p1a_kv_append: null input or negative T"); return P1A_E_ARG; }
+    if (T == 0) return P1A_OK;
+    if ((((uintptr_t) k | (uintptr_t) v) & 15) || (c->Hkv * c->D) % 32) { set_error("p1a_kv_append: k/v must be 16-byte aligned, Hkv*D %% 32 == 0"); return P1A_E_SHAPE; }
+    if (T > 65535) { set_error("p1a_kv_append: T=%d exceeds 65535 rows per call", T); return P1A_E_SHAPE; }
+    if (!pos_rows && !p0_dev && p0 < 0) { set_error("p1a_kv_append: negative p0"); return P1A_E_ARG; }
+    return launch_append(*c, k, v, p0, p0_dev, pos_rows, T, (hipStream_t) stream);
+}
+
+int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float * gate, int T, int p0,
+                    const int32_t * p0_dev, const int32_t * pos_rows, int rows_per_seq, int Hq, float scale,
+                    void * stream) {
+    if (!kv_ok(c, "p1a_attn_decode")) return P1A_E_ARG;
+    if (!q || !out) { set_error("p1a_attn_decode: null q/out"); return P1A_E_ARG; }
+    if (T < 1 || T > P1A_MAX_ROWS || Hq < c->Hkv || Hq % c->Hkv) {
+        set_error("p1a_attn_decode: unsupported shape (D=%d Hq=%d Hkv=%d T=%d)", c->D, Hq, c->Hkv, T);
+        return P1A_E_SHAPE;
+    }
+    if ((((uintptr_t) q | (uintptr_t) out | (uintptr_t) gate) & 15)) { set_error("p1a_attn_decode: q/out/gate must be 16-byte aligned"); return P1A_E_SHAPE; }
+    if (!pos_rows && !p0_dev && p0 < 0) { set_error("p1a_attn_decode: negative p0"); return P1A_E_ARG; }
+    hipStream_t s = (hipStream_t) stream;
+    decode_args a;
+    a.q = q; a.out = out; a.gate = gate; a.T = T; a.p0 = p0; a.p0_dev = p0_dev; a.pos_rows = pos_rows;
+    a.Hq = Hq; a.scale = scale;
+    a.rows_per_group = decode_rows_per_group(*c, Hq, pos_rows ? (rows_per_seq < 1 ? 1 : rows_per_seq) : T);
+    // a sequence's rows must split into whole groups, or a group would mix two sequences
+    while (pos_rows && rows_per_seq > 1 && rows_per_seq % a.rows_per_group) --a.rows_per_group;
+    a.nsplit = nsplit_for(*c, Hq);
+    const size_t NS = (size_t) a.nsplit * decode_streams_per_split(*c, Hq);
+    const size_t rows = (size_t) (T < 8 ? 8 : T) * Hq;
+    scratch * sc = scratch_for(s, rows * NS * c->D * sizeof(float), rows * NS * 2 * sizeof(float));
+    if (!sc) return P1A_E_SCRATCH;
+    a.part_o = sc->o; a.part_ml = sc->ml;
+    return launch_decode(*c, a, s);
+}
+
+int p1a_warmup(int rows, int Hq, int Hkv, int D, void * stream) {
+    if (rows < 1 || rows > P1A_MAX_ROWS || Hq < 1 || Hkv < 1 || Hq % Hkv || D < 32) { set_error("p1a_warmup: bad shape"); return P1A_E_ARG; }
+    // the largest per-row footprint over the kernels a (Hq, Hkv, D) cache can take: the generic path with 4 streams
+    p1a_kv c;
+    memset(&c, 0, sizeof c);
+    c.type = P1A_KV_Q4_0; c.Hkv = Hkv; c.D = D;
+    size_t NS = (size_t) nsplit_for(c, Hq) * 4;
+    c.type = P1A_KV_Q8_0; c.k = c.v = (void *) 16;
+    const size_t NS2 = (size_t) nsplit_for(c, Hq) * decode_streams_per_split(c, Hq);
+    if (NS2 > NS) NS = NS2;
+    const size_t r = (size_t) (rows < 8 ? 8 : rows) * Hq;
+    return scratch_for((hipStream_t) stream, r * NS * D * sizeof(float), r * NS * 2 * sizeof(float)) ? P1A_OK : P1A_E_SCRATCH;
+}
+
+int p1a_attn_prefill(const float * q, const p1a_kv * c, float * out, const float * gate, int T, int p0, int Hq,
+                     float scale, void * scratch, size_t scratch_bytes, void * stream) {
+    if (!kv_ok(c, "p1a_attn_prefill")) return P1A_E_ARG;
+    if (!q || !out || T < 1 || p0 < 0) { set_error("p1a_attn_prefill: bad argument"); return P1A_E_ARG; }
+    if (Hq < c->Hkv || Hq % c->Hkv) { set_error("p1a_attn_prefill: unsupported shape (Hq=%d Hkv=%d)", Hq, c->Hkv); return P1A_E_SHAPE; }
+    if ((((uintptr_t) q | (uintptr_t) out | (uintptr_t) gate) & 15)) { set_error("p1a_attn_prefill: q/out/gate must be 16-byte aligned"); return P1A_E_SHAPE; }
+    return launch_prefill(*c, q, out, gate, T, p0, Hq, scale, scratch, scratch_bytes, (hipStream_t) stream);
+}
+
+int p1a_sigmoid_mul(float * x, const float * g, size_t n, void * stream) {
+    if (!x || !g) { set_error("p1a_sigmoid_mul: null argument"); return P1A_E_ARG; }
+    if (!n) return P1A_OK;
+    return launch_sigmoid_mul(x, g, n, (hipStream_t) stream);
+}
+
+int p1a_get_nsplit(int Hkv) {
+    p1a_kv c;
+    memset(&c, 0, sizeof c);
+    c.type = P1A_KV_Q8_0; c.Hkv = Hkv < 1 ? 1 : Hkv; c.D = 256; c.k = c.v = (void *) 16;
+    return nsplit_for(c, 6 * c.Hkv);
+}
+
+void p1a_set_nsplit(int n) { g_nsplit_override = n > 0 ? n : 0; }
+
+void p1a_release(void) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    int cur = 0;
+    (void) hipGetDevice(&cur);
+    for (int i = 0; i < g_nscr; ++i) {
+        if (!g_scr[i].o) continue;
+        (void) hipSetDevice(g_scr[i].dev);
+        (void) hipDeviceSynchronize();
+        (void) hipFree(g_scr[i].o);
+        (void) hipFree(g_scr[i].ml);
+        g_scr[i] = scratch{};
+    }
+    g_nscr = 0;
+    (void) hipSetDevice(cur);
+}
+
+const char * p1a_last_error(void) { return g_err; }
+const char * p1a_version(void) { return "p1a_attn 0.1 (gfx950)"; }
+
+}   // extern "C"

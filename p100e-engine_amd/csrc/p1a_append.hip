@@ -1,0 +1,124 @@
+// Quantize-on-append KV write for gfx950: f32 K/V rows -> f16 / q8_0 / q4_0 cache rows, paged or contiguous.
+// The arithmetic is the reference's (src/fast/kv_q8.cuh:20-49 = ggml quantize_row_q8_0_ref / quantize_row_q4_0_ref)
+// and must stay bit-exact: this file is compiled with -ffp-contract=off, because x * id + 8.5f must round the product
+// and the sum separately, and uses IEEE division for amax / 127 and 1 / d.
+// Mapping: one lane owns 4 consecutive values (one 16-byte load for K, one for V), 8 lanes own a 32-value block and
+// reduce over it with three xor-shuffles; a 256-thread workgroup covers 1024 values of one position row.
+#include "p1a_common.hpp"
+
+#pragma clang fp contract(off)
+
+namespace p1a {
+namespace {
+
+__device__ __forceinline__ float xor8_max(float a) {
+    a = fmaxf(a, __shfl_xor(a, 1));
+    a = fmaxf(a, __shfl_xor(a, 2));
+    a = fmaxf(a, __shfl_xor(a, 4));
+    return a;
+}
+
+__device__ __forceinline__ uint16_t f16_bits(float f) {
+    const half_t h = (half_t) f;   // v_cvt_f16_f32, round-to-nearest-even
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+// q8_0 block: head = first byte of the (position, kv head) row, b = block index, nb = blocks per head
+__device__ __forceinline__ void q8_block(const float4 x, int j, char * head, int b, int nb) {
+    const float amax = xor8_max(fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w))));
+    const float d = amax / 127.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const int q0 = (int) roundf(x.x * id), q1 = (int) roundf(x.y * id), q2 = (int) roundf(x.z * id), q3 = (int) roundf(x.w * id);
+    const uint32_t w = (uint32_t) (q0 & 0xff) | ((uint32_t) (q1 & 0xff) << 8) | ((uint32_t) (q2 & 0xff) << 16) | ((uint32_t) (q3 & 0xff) << 24);
+    *reinterpret_cast<uint32_t *>(head + nb * 2 + b * 32 + j * 4) = w;
+    if (j == 0) *reinterpret_cast<uint16_t *>(head + b * 2) = f16_bits(d);
+}
+
+// q4_0 block: blk = the 18-byte ggml block
+__device__ __forceinline__ void q4_block(const float4 x, int j, char * blk) {
+    // signed value of largest magnitude, first index on ties (strict > keeps the earlier one)
+    float a = fabsf(x.x), xm = x.x;
+    int idx = 4 * j;
+    if (fabsf(x.y) > a) { a = fabsf(x.y); xm = x.y; idx = 4 * j + 1; }
+    if (fabsf(x.z) > a) { a = fabsf(x.z); xm = x.z; idx = 4 * j + 2; }
+    if (fabsf(x.w) > a) { a = fabsf(x.w); xm = x.w; idx = 4 * j + 3; }
+#pragma unroll
+    for (int o = 1; o < 8; o <<= 1) {
+        const float oa = __shfl_xor(a, o), ox = __shfl_xor(xm, o);
+        const int oi = __shfl_xor(idx, o);
+        if (oa > a || (oa == a && oi < idx)) { a = oa; xm = ox; idx = oi; }
+    }
+    const float mx = a > 0.0f ? xm : 0.0f;
+    const float d = mx / -8.0f;
+    const float id = d != 0.0f ? 1.0f / d : 0.0f;
+    const float p0 = x.x * id, p1 = x.y * id, p2 = x.z * id, p3 = x.w * id;   // rounded products
+    const int q0 = min(15, (int) (p0 + 8.5f)), q1 = min(15, (int) (p1 + 8.5f));
+    const int q2 = min(15, (int) (p2 + 8.5f)), q3 = min(15, (int) (p3 + 8.5f));
+    const int mine = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
+    const int hi = __shfl_down(mine, 4);   // lanes 4..7 of the block hold values 16..31 = the high nibbles
+    if (j < 4) {
+        const uint32_t w = (uint32_t) mine | ((uint32_t) hi << 4);
+        uint16_t * dst = reinterpret_cast<uint16_t *>(blk + 2 + 4 * j);   // 2-byte aligned only
+        dst[0] = (uint16_t) w;
+        dst[1] = (uint16_t) (w >> 16);
+    }
+    if (j == 0) *reinterpret_cast<uint16_t *>(blk) = f16_bits(d);
+}
+
+template <uint32_t KT>
+__global__ void __launch_bounds__(256) append_k(const float * __restrict__ k, const float * __restrict__ v, char * kc,
+                                                char * vc, int p0, const int32_t * __restrict__ p0_dev,
+                                                const int32_t * __restrict__ pos_rows, int Hkv, int D, kv_view pg) {
+    const int t = blockIdx.y;
+    const int i4 = blockIdx.x * 256 + threadIdx.x;   // index of this lane's 4 values within the row
+    const int n4 = Hkv * D / 4;
+    // lanes past the row still take part in the shuffles of their (non-existent) block; n4 % 8 == 0 so a block is
+    // never split between live and dead lanes
+    const bool live = i4 < n4;
+    int pos;
+    if (pos_rows) pos = pos_rows[t];
+    else pos = (p0_dev ? *p0_dev : p0) + t;
+    const size_t o = kv_off_tab(pg, kv_tab(pg, pos_rows ? t : 0), pos);
+    float4 xk = make_float4(0.f, 0.f, 0.f, 0.f), xv = xk;
+    if (live) {
+        xk = reinterpret_cast<const float4 *>(k + (size_t) t * Hkv * D)[i4];
+        xv = reinterpret_cast<const float4 *>(v + (size_t) t * Hkv * D)[i4];
+    }
+    if constexpr (KT == P1A_KV_F16) {
+        if (live) {
+            h4 hk = {(half_t) xk.x, (half_t) xk.y, (half_t) xk.z, (half_t) xk.w};
+            h4 hv = {(half_t) xv.x, (half_t) xv.y, (half_t) xv.z, (half_t) xv.w};
+            reinterpret_cast<h4 *>(kc + o)[i4] = hk;
+            reinterpret_cast<h4 *>(vc + o)[i4] = hv;
+        }
+    } else {
+        const int nb = D / 32;
+        const int blk = i4 >> 3, j = i4 & 7;   // block over Hkv * nb, lane within the block
+        const int h = blk / nb, b = blk - h * nb;
+        if constexpr (KT == P1A_KV_Q8_0) {
+            const size_t ho = o + (size_t) h * nb * 34;
+            if (live) { q8_block(xk, j, kc + ho, b, nb); q8_block(xv, j, vc + ho, b, nb); }
+            else { xor8_max(0.f); xor8_max(0.f); }
+        } else {
+            const size_t bo = o + (size_t) blk * 18;
+            // dead lanes form whole 8-lane groups, so the live groups' shuffles never read them
+            if (live) { q4_block(xk, j, kc + bo); q4_block(xv, j, vc + bo); }
+        }
+    }
+}
+
+}   // namespace
+
+int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, const int32_t * p0_dev,
+                  const int32_t * pos_rows, int T, hipStream_t s) {
+    const kv_view pg = view_of(c);
+    const int n4 = c.Hkv * c.D / 4;
+    const dim3 grid((n4 + 255) / 256, T);
+    char * kc = (char *) c.k, * vc = (char *) c.v;
+    if (c.type == P1A_KV_F16) append_k<P1A_KV_F16><<<grid, 256, 0, s>>>(k, v, kc, vc, p0, p0_dev, pos_rows, c.Hkv, c.D, pg);
+    else if (c.type == P1A_KV_Q8_0) append_k<P1A_KV_Q8_0><<<grid, 256, 0, s>>>(k, v, kc, vc, p0, p0_dev, pos_rows, c.Hkv, c.D, pg);
+    else append_k<P1A_KV_Q4_0><<<grid, 256, 0, s>>>(k, v, kc, vc, p0, p0_dev, pos_rows, c.Hkv, c.D, pg);
+    return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
+}
+
+}   // namespace p1a

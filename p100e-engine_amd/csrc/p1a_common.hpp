@@ -1,0 +1,74 @@
+// Shared device/host helpers of the gfx950 paged-KV attention library (internal header).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <cstddef>
+#include <cstdint>
+#include "p1a_attn.h"
+
+namespace p1a {
+
+typedef _Float16 half_t;
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f16x __attribute__((ext_vector_type(16)));
+typedef int i2 __attribute__((ext_vector_type(2)));
+typedef int i4 __attribute__((ext_vector_type(4)));
+typedef short s4 __attribute__((ext_vector_type(4)));
+
+// Paged addressing: the device twin of the reference's kv_pg helpers (src/fast/kv_page.cuh:11-31), with 64-bit
+// page bases throughout.
+struct kv_view {
+    const int32_t * pt;     // page table(s); nullptr = contiguous
+    const int32_t * rtab;   // per-row element offsets into pt; nullptr = 0
+    int psh;
+    size_t pstride;
+    size_t rowb;            // bytes of one position (all kv heads)
+};
+
+inline kv_view view_of(const p1a_kv & c) {
+    return kv_view{c.pt, c.rtab, c.psh, c.pstride, p1a_kv_row_bytes(c.type, c.Hkv, c.D)};
+}
+
+__device__ __forceinline__ const int32_t * kv_tab(const kv_view & g, int t) {
+    return g.pt ? (g.rtab ? g.pt + g.rtab[t] : g.pt) : nullptr;
+}
+__device__ __forceinline__ size_t kv_off_tab(const kv_view & g, const int32_t * tab, int p) {
+    if (!tab) return (size_t) p * g.rowb;
+    return (size_t) tab[p >> g.psh] * g.pstride + (size_t) (p & ((1 << g.psh) - 1)) * g.rowb;
+}
+
+constexpr size_t head_bytes(uint32_t type, int D) {
+    return type == P1A_KV_F16 ? (size_t) D * 2 : type == P1A_KV_Q8_0 ? (size_t) (D / 32) * 34 : (size_t) (D / 32) * 18;
+}
+
+// host-side launch entry points implemented in the .hip files
+int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, const int32_t * p0_dev,
+                  const int32_t * pos_rows, int T, hipStream_t s);
+
+struct decode_args {
+    const float * q;
+    float * out;
+    const float * gate;
+    int T, p0;
+    const int32_t * p0_dev;
+    const int32_t * pos_rows;
+    int rows_per_group;   // rows sharing one KV read
+    int Hq;
+    float scale;
+    int nsplit;
+    float * part_o;       // [T*Hq][nsplit][D]
+    float * part_ml;      // [T*Hq][nsplit][2]
+};
+int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s);
+int decode_streams_per_split(const p1a_kv & c, int Hq);
+int decode_default_nsplit(const p1a_kv & c, int Hq, int cus);
+int decode_rows_per_group(const p1a_kv & c, int Hq, int want);
+int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
+                   float scale, void * scratch, size_t scratch_bytes, hipStream_t s);
+int launch_sigmoid_mul(float * x, const float * g, size_t n, hipStream_t s);
+
+void set_error(const char * fmt, ...);
+
+}   // namespace p1a

@@ -1,0 +1,48 @@
+"""The C-ABI library loads without a GPU and exports every function include/*.h declares; refusals launch nothing."""
+import ctypes
+import glob
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared():
+    names = []
+    for h in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(h).read(), flags=re.S)
+        names += re.findall(r"\b(p1a_[a-z0-9_]+)\s*\(", text)
+    return sorted(set(names))
+
+
+def test_exports_match_header(p1a):
+    names = declared()
+    assert len(names) >= 10
+    L = ctypes.CDLL(p1a.lib_path())
+    for n in names:
+        assert hasattr(L, n), n
+    assert sorted(p1a.EXPORTS) == names
+
+
+def test_row_bytes_and_version(p1a):
+    assert p1a.kv_row_bytes(p1a.KV_F16, 4, 256) == 2048
+    assert p1a.kv_row_bytes(p1a.KV_Q8_0, 4, 256) == 1088
+    assert p1a.kv_row_bytes(p1a.KV_Q4_0, 4, 256) == 576
+    assert b"gfx950" in p1a.lib().p1a_version()
+
+
+def test_refusals_do_not_launch(p1a):
+    # argument validation happens before any HIP call, so it can be exercised without a GPU
+    from importlib import import_module
+    b = import_module("p100e-engine_amd.binding")
+    kv = b.p1a_kv()
+    L = p1a.lib()
+    assert L.p1a_kv_append(ctypes.byref(kv), None, None, 0, None, None, 1, None) == -2      # null cache
+    kv.k = kv.v = 4096
+    kv.type, kv.Hkv, kv.D = 77, 4, 256
+    assert L.p1a_attn_decode(4096, ctypes.byref(kv), 4096, None, 1, 0, None, None, 0, 24, 0.0625, None) == -2   # unknown type
+    kv.type = p1a.KV_Q8_0
+    assert L.p1a_attn_decode(4096, ctypes.byref(kv), 4096, None, 1, 0, None, None, 0, 25, 0.0625, None) == -1   # Hq % Hkv
+    assert L.p1a_attn_decode(4096, ctypes.byref(kv), 4096, None, 33, 0, None, None, 0, 24, 0.0625, None) == -1  # too many rows
+    assert L.p1a_attn_decode(4100, ctypes.byref(kv), 4096, None, 1, 0, None, None, 0, 24, 0.0625, None) == -1   # misaligned q
+    assert b"aligned" in L.p1a_last_error()
