@@ -1,0 +1,159 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged-KV attention hot path on one MI355X.
+
+Workload (N = 1): BASELINE.json configs[1] - 27B-shape decode, batch 1, one full-attention layer: 24 q heads / 4 kv
+heads, head_dim 256, context 32768, q8_0 KV in 256-token pages scattered by a random permutation page table, fused
+sigmoid gate. A "step" is one p1a_attn_decode call (split-K kernel + merge) on inputs resident in HBM. The K timed
+steps are captured once into a hipGraph (the engine replays its decode step as a graph as well) and walk over several
+distinct KV pools, so that consecutive steps do not find their 71 MB of KV in the 256 MB Infinity Cache.
+
+Prints ONE JSON line: metric / value (GB/s of algorithmic KV bytes) plus `roofline` and `cpu_baseline` objects, and
+secondary measurements (same-pool rate, verify, batched decode, prefill, append) under `extra`.
+"""
+import argparse
+import ctypes
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def build_pool(p1a, torch, kv_type, Hq, Hkv, D, psh, n_ctx, n_seq, seed):
+    """n_seq sequences of n_ctx tokens in one paged pool, page tables a random permutation; K/V are N(0,1), K
+    RMS-normed per head, written through the library's own quantize-on-append."""
+    ps = 1 << psh
+    ppseq = (n_ctx + ps - 1) // ps
+    n_pages = ppseq * n_seq
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    perm = torch.randperm(n_pages, generator=g, device="cuda").to(torch.int32)
+    tabs = perm.reshape(ppseq, n_seq).t().contiguous().reshape(-1)       # pages interleaved across the slots
+    kv = p1a.KVCache.paged(kv_type, Hkv, D, psh, n_pages, tabs, ppseq)
+    chunk = 4096
+    for s in range(n_seq):
+        c = kv.slot(s, ppseq)
+        for a in range(0, n_ctx, chunk):
+            T = min(chunk, n_ctx - a)
+            k = torch.randn((T, Hkv, D), generator=g, device="cuda")
+            k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + 1e-6)
+            v = torch.randn((T, Hkv, D), generator=g, device="cuda")
+            p1a.kv_append(c, k, v, a, T)
+    torch.cuda.synchronize()
+    return kv, ppseq
+
+
+def time_graph(torch, stream, fn_list, warmup):
+    """capture the calls of fn_list into one graph on `stream`, replay `warmup` times, then time one replay with
+    events recorded on that same stream. Returns seconds per call."""
+    with torch.cuda.stream(stream):
+        for f in fn_list[:2]:
+            f()
+        stream.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for f in fn_list:
+                f()
+        for _ in range(max(1, warmup)):
+            g.replay()
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        g.replay()
+        e1.record(stream)
+        e1.synchronize()
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / len(fn_list)
+
+
+def cpu_baseline(Hq, Hkv, D, n_ctx, seed):
+    """The CPU oracle (fp32 restatement of the reference's attention kernel) on a bounded sample of the same
+    workload: one query row over a q8_0 cache of n_ctx tokens, repeated for about 10 s."""
+    import numpy as np
+    import _inputs as I
+    import _oracle as O
+    q, k, v, gate = I.qkv(seed, n_ctx, 1, Hq, Hkv, D)
+    c = O.HostKV.contiguous(O.KV_Q8_0, n_ctx, Hkv, D)
+    O.kv_append_rows(c, k, v, np.arange(n_ctx))
+    pos = np.array([n_ctx - 1], np.int32)
+    O.attn_rows(c, q, pos, Hq, 1.0 / 16, gate=gate)
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        out = O.attn_rows(c, q, pos, Hq, 1.0 / 16, gate=gate)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > 10.0 or reps >= 50:
+            break
+    bytes_ = 2 * n_ctx * O.row_bytes(O.KV_Q8_0, Hkv, D)
+    return {"value": bytes_ * reps / dt / 1e9, "unit": "GB/s", "cores": int(O.lib().orc_num_threads()), "kind": "port",
+            "sample": f"{reps} full decode steps (1 row, ctx {n_ctx}, q8_0) of the C oracle with OpenMP, {dt:.1f} s"}, out, (q, gate, c)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on ONE GPU only (no collectives are part of it); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    p1a = importlib.import_module("p100e-engine_amd")
+    p1a.lib()
+    Hq, Hkv, D, psh, n_ctx = 24, 4, 256, 8, 32768
+    scale = 1.0 / 16.0
+    rowb = p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
+    step_bytes = 2 * n_ctx * rowb                                          # K + V of the visible positions
+    n_pools = 8                                                            # 8 x 71 MB > 256 MB Infinity Cache
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, n_ctx, n_pools, seed=1234)
+    g = torch.Generator(device="cuda").manual_seed(99)
+    q = torch.randn((1, Hq, D), generator=g, device="cuda")
+    q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + 1e-6)
+    gate = torch.randn((1, Hq * D), generator=g, device="cuda")
+    out = torch.empty((1, Hq, D), device="cuda")
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        p1a.warmup(32, Hq, Hkv, D)
+    slots = [kv.slot(s, ppseq) for s in range(n_pools)]
+
+    def step(i):
+        return lambda: p1a.attn_decode(q, slots[i % n_pools], out, 1, n_ctx - 1, Hq, scale, gate=gate)
+
+    K, W = args.steps, args.warmup
+    torch.cuda.synchronize()
+    sec = time_graph(torch, stream, [step(i) for i in range(K)], W)
+    sec_same = time_graph(torch, stream, [step(0) for _ in range(K)], W)
+    gbs = step_bytes / sec / 1e9
+    res = {
+        "metric": "decode-attn HBM GB/s @27B q8_0 32K (paged, B=1, fused gate)", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "q8_0 KV -> f16 MFMA, f32 accumulate", "data": "synthetic",
+        "config": {"workload": "configs[1]: decode 24/4 heads, head_dim 256, ctx 32768, q8_0, 256-token pages, random page table",
+                   "kv_bytes_per_step": step_bytes, "pools_rotated": n_pools, "launch": "hipGraph of K steps"},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "note": "achieved = KV bytes / whole step (split-K kernel + merge kernel), event-timed"},
+        "extra": {"same_pool_GBs": round(step_bytes / sec_same / 1e9, 1), "same_pool_us": round(sec_same * 1e6, 2),
+                  "nsplit": p1a.get_nsplit(Hkv)},
+    }
+    if not args.no_cpu:
+        cb, ref, (hq, hgate, hc) = cpu_baseline(Hq, Hkv, D, n_ctx, seed=7)
+        res["cpu_baseline"] = cb
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()

@@ -78,11 +78,10 @@ bool kv_ok(const p1a_kv * c, const char * who) {
     return true;
 }
 
-int nsplit_for(const p1a_kv & c, int Hq) {
+// requested split-stream count: the setter, then the environment, else 0 = the plan's default for the device
+int nsplit_req() {
     static const int env = getenv("P1A_DEC_SPLIT") ? atoi(getenv("P1A_DEC_SPLIT")) : 0;
-    if (g_nsplit_override > 0) return g_nsplit_override;
-    if (env > 0) return env;
-    return decode_default_nsplit(c, Hq, cu_count());
+    return g_nsplit_override > 0 ? g_nsplit_override : (env > 0 ? env : 0);
 }
 
 }   // namespace
@@ -125,10 +124,11 @@ int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float 
     a.rows_per_group = decode_rows_per_group(*c, Hq, pos_rows ? (rows_per_seq < 1 ? 1 : rows_per_seq) : T);
     // a sequence's rows must split into whole groups, or a group would mix two sequences
     while (pos_rows && rows_per_seq > 1 && rows_per_seq % a.rows_per_group) --a.rows_per_group;
-    a.nsplit = nsplit_for(*c, Hq);
-    const size_t NS = (size_t) a.nsplit * decode_streams_per_split(*c, Hq);
-    const size_t rows = (size_t) (T < 8 ? 8 : T) * Hq;
-    scratch * sc = scratch_for(s, rows * NS * c->D * sizeof(float), rows * NS * 2 * sizeof(float));
+    a.nsplit = nsplit_req();
+    a.cus = cu_count();
+    size_t need_o, need_ml;
+    decode_scratch_need(*c, Hq, T < 8 ? 8 : T, a.rows_per_group, a.nsplit, a.cus, need_o, need_ml);
+    scratch * sc = scratch_for(s, need_o, need_ml);
     if (!sc) return P1A_E_SCRATCH;
     a.part_o = sc->o; a.part_ml = sc->ml;
     return launch_decode(*c, a, s);
@@ -136,16 +136,21 @@ int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float 
 
 int p1a_warmup(int rows, int Hq, int Hkv, int D, void * stream) {
     if (rows < 1 || rows > P1A_MAX_ROWS || Hq < 1 || Hkv < 1 || Hq % Hkv || D < 32) { set_error("p1a_warmup: bad shape"); return P1A_E_ARG; }
-    // the largest per-row footprint over the kernels a (Hq, Hkv, D) cache can take: the generic path with 4 streams
+    // the largest footprint over the kernels and row groupings a (Hq, Hkv, D) cache can take
     p1a_kv c;
     memset(&c, 0, sizeof c);
-    c.type = P1A_KV_Q4_0; c.Hkv = Hkv; c.D = D;
-    size_t NS = (size_t) nsplit_for(c, Hq) * 4;
-    c.type = P1A_KV_Q8_0; c.k = c.v = (void *) 16;
-    const size_t NS2 = (size_t) nsplit_for(c, Hq) * decode_streams_per_split(c, Hq);
-    if (NS2 > NS) NS = NS2;
-    const size_t r = (size_t) (rows < 8 ? 8 : rows) * Hq;
-    return scratch_for((hipStream_t) stream, r * NS * D * sizeof(float), r * NS * 2 * sizeof(float)) ? P1A_OK : P1A_E_SCRATCH;
+    c.Hkv = Hkv; c.D = D; c.k = c.v = (void *) 16;
+    size_t need_o = 0, need_ml = 0;
+    const uint32_t types[3] = {P1A_KV_F16, P1A_KV_Q8_0, P1A_KV_Q4_0};
+    for (uint32_t ty : types)
+        for (int rg = 1; rg <= 4; ++rg) {
+            size_t o, m;
+            c.type = ty;
+            decode_scratch_need(c, Hq, rows < 8 ? 8 : rows, rg, nsplit_req(), cu_count(), o, m);
+            if (o > need_o) need_o = o;
+            if (m > need_ml) need_ml = m;
+        }
+    return scratch_for((hipStream_t) stream, need_o, need_ml) ? P1A_OK : P1A_E_SCRATCH;
 }
 
 int p1a_attn_prefill(const float * q, const p1a_kv * c, float * out, const float * gate, int T, int p0, int Hq,
@@ -167,7 +172,7 @@ int p1a_get_nsplit(int Hkv) {
     p1a_kv c;
     memset(&c, 0, sizeof c);
     c.type = P1A_KV_Q8_0; c.Hkv = Hkv < 1 ? 1 : Hkv; c.D = 256; c.k = c.v = (void *) 16;
-    return nsplit_for(c, 6 * c.Hkv);
+    return decode_nsplit(c, 6 * c.Hkv, nsplit_req(), cu_count());
 }
 
 void p1a_set_nsplit(int n) { g_nsplit_override = n > 0 ? n : 0; }

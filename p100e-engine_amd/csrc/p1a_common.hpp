@@ -16,6 +16,7 @@ typedef float f16x __attribute__((ext_vector_type(16)));
 typedef int i2 __attribute__((ext_vector_type(2)));
 typedef int i4 __attribute__((ext_vector_type(4)));
 typedef short s4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
 
 // Paged addressing: the device twin of the reference's kv_pg helpers (src/fast/kv_page.cuh:11-31), with 64-bit
 // page bases throughout.
@@ -57,14 +58,16 @@ struct decode_args {
     int rows_per_group;   // rows sharing one KV read
     int Hq;
     float scale;
-    int nsplit;
+    int nsplit;           // requested split streams (0 = default for the device)
+    int cus;              // compute units of the device
     float * part_o;       // [T*Hq][nsplit][D]
     float * part_ml;      // [T*Hq][nsplit][2]
 };
 int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s);
-int decode_streams_per_split(const p1a_kv & c, int Hq);
-int decode_default_nsplit(const p1a_kv & c, int Hq, int cus);
 int decode_rows_per_group(const p1a_kv & c, int Hq, int want);
+int decode_nsplit(const p1a_kv & c, int Hq, int nsplit_req, int cus);
+void decode_scratch_need(const p1a_kv & c, int Hq, int rows, int rows_per_group, int nsplit_req, int cus,
+                         size_t & bytes_o, size_t & bytes_ml);
 int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s);
 int launch_sigmoid_mul(float * x, const float * g, size_t n, hipStream_t s);

@@ -1,0 +1,72 @@
+"""Helpers of the GPU parity tests: host caches built by the oracle, mirrored byte-for-byte on the device."""
+import numpy as np
+import torch
+
+import _inputs as I
+import _oracle as O
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+class Pool:
+    """A paged pool holding several sequences (the engine's layout, one layer of n_layers selected), built on the
+    host by the oracle's append and copied to the device; plus each sequence's contiguous twin."""
+
+    def __init__(self, p1a, kv_type, Hq, Hkv, D, psh, lens, seed, n_layers=2, layer=1, f16_inputs=False, shuffle=True,
+                 spare_pages=3, fill="oracle"):
+        self.p1a, self.type, self.Hq, self.Hkv, self.D, self.psh = p1a, kv_type, Hq, Hkv, D, psh
+        ps = 1 << psh
+        self.lens = list(lens)
+        self.maxp = max((n + ps - 1) // ps for n in lens) + 1
+        need = sum((n + ps - 1) // ps for n in lens)
+        self.np_pages = need + spare_pages
+        g = I.rng(seed)
+        order = g.permutation(self.np_pages).astype(np.int32) if shuffle else np.arange(self.np_pages, dtype=np.int32)
+        self.tabs = np.zeros(len(lens) * self.maxp, np.int32)
+        used = 0
+        # deal pages round-robin across the sequences, so their pages interleave in the pool
+        want = [(n + ps - 1) // ps for n in lens]
+        for p in range(max(want)):
+            for s in range(len(lens)):
+                if p < want[s]:
+                    self.tabs[s * self.maxp + p] = order[used]
+                    used += 1
+        self.host = O.HostKV.paged(kv_type, Hkv, D, psh, self.np_pages, self.tabs, self.maxp, n_layers=n_layers, layer=layer)
+        self.k, self.v, self.cont = [], [], []
+        for s, n in enumerate(lens):
+            _, k, v, _ = I.qkv(seed * 131 + s, n, 1, Hq, Hkv, D, f16_inputs=f16_inputs)
+            self.k.append(k)
+            self.v.append(v)
+            if fill == "oracle":
+                O.kv_append_rows(self.host.view(rtab=np.full(n, s * self.maxp, np.int32)), k, v, np.arange(n))
+        self.dtabs = dev(self.tabs)
+        self.dpool = dev(self.host.pool)
+        self.devkv = p1a.KVCache.paged(kv_type, Hkv, D, psh, self.np_pages, self.dtabs, self.maxp, n_layers=n_layers,
+                                      layer=layer, pool=self.dpool)
+
+    def host_seq(self, s):
+        """host view of sequence s (page table row s)"""
+        return self.host.view(pt=self.tabs[s * self.maxp:])
+
+    def dev_seq(self, s):
+        return self.devkv.slot(s, self.maxp)
+
+    def host_contiguous(self, s):
+        n = self.lens[s]
+        c = O.HostKV.contiguous(self.type, n, self.Hkv, self.D)
+        O.kv_append_rows(c, self.k[s], self.v[s], np.arange(n))
+        return c
+
+    def dev_contiguous(self, s):
+        h = self.host_contiguous(s)
+        dk, dv = dev(h.k), dev(h.v)
+        return self.p1a.KVCache(self.type, self.lens[s], self.Hkv, self.D, dk.data_ptr(), dv.data_ptr(), keep=(dk, dv))
+
+
+def check(out, ref, what=""):
+    ma, rl = I.errors(out, ref)
+    assert np.all(np.isfinite(out)), what
+    assert ma <= I.MAX_ABS_TOL and rl <= I.REL_L2_TOL, f"{what}: max_abs={ma:.3e} rel_l2={rl:.3e}"
+    return ma, rl

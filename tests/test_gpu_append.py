@@ -1,0 +1,79 @@
+"""Quantize-on-append on the GPU (through the C ABI) vs the oracle: every byte must match."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import _inputs as I
+import _oracle as O
+from _gpu import Pool, dev
+
+pytestmark = pytest.mark.gpu
+TYPES = [O.KV_F16, O.KV_Q8_0, O.KV_Q4_0]
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "quant_golden.npz"))
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("Hkv,D", [(4, 256), (1, 64), (2, 128), (3, 96)])
+def test_contiguous_bytes(p1a, kv_type, Hkv, D):
+    T, p0, n_ctx = 37, 5, 48
+    g = I.rng(100 + D)
+    k = I.normal(g, (T, Hkv, D)) * 1.7
+    v = I.normal(g, (T, Hkv, D)) * 0.3
+    k[3] = 0.0                      # an all-zero row
+    v[4, :, :32] = 0.0
+    host = O.HostKV.contiguous(kv_type, n_ctx, Hkv, D)
+    O.kv_append_rows(host, k, v, p0 + np.arange(T))
+    c = p1a.KVCache.contiguous(kv_type, n_ctx, Hkv, D)
+    p1a.kv_append(c, dev(k), dev(v), p0, T)
+    torch.cuda.synchronize()
+    assert np.array_equal(c._keep[0].cpu().numpy(), host.k)
+    assert np.array_equal(c._keep[1].cpu().numpy(), host.v)
+
+
+@pytest.mark.parametrize("kv_type", [O.KV_Q8_0, O.KV_Q4_0])
+def test_golden_blocks_on_gpu(p1a, kv_type):
+    """the reference's own quantizer outputs, reproduced by the HIP kernel (edge cases included)"""
+    x = GOLD["x"]
+    n = x.shape[0] // 8 * 8
+    rows = x[:n].reshape(n // 8, 1, 256)
+    c = p1a.KVCache.contiguous(kv_type, n // 8, 1, 256)
+    p1a.kv_append(c, dev(rows), dev(rows), 0, n // 8)
+    torch.cuda.synchronize()
+    got = c._keep[0].cpu().numpy().reshape(n // 8, -1)
+    if kv_type == O.KV_Q8_0:
+        assert np.array_equal(got[:, :16].copy().view(np.uint16).reshape(-1), GOLD["q8_d"][:n])
+        assert np.array_equal(got[:, 16:].copy().view(np.int8).reshape(n, 32), GOLD["q8_q"][:n])
+    else:
+        assert np.array_equal(got.reshape(n, 18), GOLD["q4_blk"][:n])
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_paged_dev_and_rows(p1a, kv_type):
+    Hq, Hkv, D, psh = 12, 2, 256, 5
+    lens = [70, 200, 33]
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=3, n_layers=3, layer=1, fill="none")
+    # host side: oracle appends; device side: chunks via host p0, device p0, and multi-sequence rows
+    for s, n in enumerate(lens):
+        O.kv_append_rows(pool.host.view(rtab=np.full(n, s * pool.maxp, np.int32)), pool.k[s], pool.v[s], np.arange(n))
+    dk = [dev(k) for k in pool.k]
+    dv = [dev(v) for v in pool.v]
+    c0 = pool.dev_seq(0)
+    p1a.kv_append(c0, dk[0], dv[0], 0, 64)
+    p1a.kv_append(c0, dk[0][64:], dv[0][64:], 64, lens[0] - 64)
+    c1 = pool.dev_seq(1)
+    p0d = dev(np.array([0], np.int32))
+    for a in range(0, lens[1], 50):
+        p0d.fill_(a)
+        p1a.kv_append_dev(c1, dk[1][a:], dv[1][a:], p0d, min(50, lens[1] - a))
+    # rows of sequences 2, 0 (rewrite), 2 in one call
+    n2 = lens[2]
+    rows_s = [2] * n2 + [0, 0]
+    rows_p = list(range(n2)) + [10, 69]
+    kk = torch.cat([dk[2], dk[0][10:11], dk[0][69:70]])
+    vv = torch.cat([dv[2], dv[0][10:11], dv[0][69:70]])
+    cr = pool.devkv.with_rows(dev(np.array([s * pool.maxp for s in rows_s], np.int32)))
+    p1a.kv_append_rows(cr, kk, vv, dev(np.array(rows_p, np.int32)), len(rows_p))
+    torch.cuda.synchronize()
+    assert np.array_equal(pool.dpool.cpu().numpy(), pool.host.pool)

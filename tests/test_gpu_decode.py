@@ -1,0 +1,151 @@
+"""Decode / MTP-verify attention on the GPU (through the C ABI) vs the CPU oracle, plus the bitwise invariances the
+reference engine tests: paged == contiguous, row t of a T-row call == the T = 1 call, rows == single, device p0 ==
+host p0. Tolerance of the path: max-abs 2e-3, rel-L2 1e-3 vs the fp32 oracle."""
+import numpy as np
+import pytest
+import torch
+
+import _inputs as I
+import _oracle as O
+from _gpu import Pool, check, dev
+
+pytestmark = pytest.mark.gpu
+TYPES = [O.KV_F16, O.KV_Q8_0, O.KV_Q4_0]
+
+
+def run_decode(p1a, c, q, T, p0, Hq, scale, gate=None):
+    out = torch.full((T, Hq, c.D), float("nan"), device="cuda")
+    p1a.attn_decode(dev(q), c, out, T, p0, Hq, scale, gate=None if gate is None else dev(gate))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def test_config1_tiny_f16(p1a):
+    """1 sequence, 4 q heads / 1 kv head, D 64, ctx 512, f16 KV in 16-token pages, identity table, scale 1/8, seed 0"""
+    Hq, Hkv, D, n = 4, 1, 64, 512
+    pool = Pool(p1a, O.KV_F16, Hq, Hkv, D, 4, [n], seed=0, n_layers=1, layer=0, f16_inputs=True, shuffle=False, spare_pages=0)
+    assert np.array_equal(pool.tabs[:32], np.arange(32))
+    q, _, _, _ = I.qkv(0, n, 1, Hq, Hkv, D, f16_inputs=True)
+    ref = O.attn_rows(pool.host_seq(0), q, np.array([n - 1]), Hq, 0.125)
+    out = run_decode(p1a, pool.dev_seq(0), q, 1, n - 1, Hq, 0.125)
+    check(out, ref, "config 1")
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_decode_vs_oracle_paged(p1a, kv_type):
+    Hq, Hkv, D, psh = 24, 4, 256, 8
+    lens = [3000, 700]
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=17)
+    scale = 1.0 / 16.0
+    for s, p0, T in [(0, 2999, 1), (0, 2045, 4), (1, 0, 1), (1, 255, 2), (1, 256, 3), (0, 31, 1), (0, 32, 1), (1, 696, 4)]:
+        q, _, _, gate = I.qkv(1000 + p0, 1, T, Hq, Hkv, D)
+        pos = p0 + np.arange(T, dtype=np.int32)
+        ref = O.attn_rows(pool.host_seq(s), q, pos, Hq, scale, gate=gate)
+        out = run_decode(p1a, pool.dev_seq(s), q, T, p0, Hq, scale, gate=gate)
+        check(out, ref, f"type {kv_type} seq {s} p0 {p0} T {T}")
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_bitwise_invariances(p1a, kv_type):
+    Hq, Hkv, D, psh = 12, 2, 256, 5
+    lens = [700, 1500, 300]
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=5, n_layers=2, layer=1)
+    scale = 1.0 / 16.0
+    q = I.normal(I.rng(77), (8, Hq, D)) * 1.5
+    dq = dev(q)
+    conts = [pool.dev_contiguous(s) for s in range(3)]
+    # paged == contiguous and T-invariance, host p0 and device p0
+    p0d = dev(np.array([0], np.int32))
+    for s in range(3):
+        for T in (1, 2, 3, 4, 7):
+            for p0 in (0, 1, 31, 32, 127, 128, 255, 256, 257, 511, 600, lens[s] - T):
+                if p0 < 0 or p0 + T > lens[s]:
+                    continue
+                a = torch.empty((T, Hq, D), device="cuda")
+                b = torch.empty((T, Hq, D), device="cuda")
+                d = torch.empty((T, Hq, D), device="cuda")
+                p1a.attn_decode(dq, conts[s], a, T, p0, Hq, scale)
+                p1a.attn_decode(dq, pool.dev_seq(s), b, T, p0, Hq, scale)
+                p0d.fill_(p0)
+                p1a.attn_decode_dev(dq, pool.dev_seq(s), d, T, p0d, lens[s], Hq, scale)
+                assert torch.equal(a, b), (s, T, p0)
+                assert torch.equal(a, d), (s, T, p0)
+                for t in range(T):
+                    one = torch.empty((1, Hq, D), device="cuda")
+                    p1a.attn_decode(dq[t:t + 1], conts[s], one, 1, p0 + t, Hq, scale)
+                    assert torch.equal(one[0], a[t]), (s, T, p0, t)
+    # multi-row: rows of 3 sequences in one call == T = 1 per row on the contiguous caches
+    sets = [
+        [(0, 699)],
+        [(0, 699), (1, 1499), (2, 299)],
+        [(1, 1099), (0, 600), (1, 900), (2, 250), (1, 430)],
+        [(0, 650), (0, 651), (1, 1496), (1, 1497), (1, 1498), (2, 100), (2, 101), (2, 102)],
+        [(2, 0), (0, 0), (1, 255), (1, 256), (0, 31), (0, 32)],
+    ]
+    for rows in sets:
+        T = len(rows)
+        pos = dev(np.array([p for _, p in rows], np.int32))
+        rt = dev(np.array([s * pool.maxp for s, _ in rows], np.int32))
+        out = torch.empty((T, Hq, D), device="cuda")
+        p1a.attn_decode_rows(dq, pool.devkv.with_rows(rt), out, T, pos, Hq, scale)
+        for t, (s, p) in enumerate(rows):
+            one = torch.empty((1, Hq, D), device="cuda")
+            p1a.attn_decode(dq[t:t + 1], conts[s], one, 1, p, Hq, scale)
+            assert torch.equal(one[0], out[t]), (rows, t)
+    # verify blocks of several sequences sharing their KV read: 3 sequences x 2 rows
+    rows = [(0, 650), (0, 651), (1, 1496), (1, 1497), (2, 100), (2, 101)]
+    pos = dev(np.array([p for _, p in rows], np.int32))
+    rt = dev(np.array([s * pool.maxp for s, _ in rows], np.int32))
+    out = torch.empty((6, Hq, D), device="cuda")
+    p1a.attn_decode_rows(dq, pool.devkv.with_rows(rt), out, 6, pos, Hq, scale, rows_per_seq=2)
+    for t, (s, p) in enumerate(rows):
+        one = torch.empty((1, Hq, D), device="cuda")
+        p1a.attn_decode(dq[t:t + 1], conts[s], one, 1, p, Hq, scale)
+        assert torch.equal(one[0], out[t]), ("blocks", t)
+
+
+def test_config3_batched_slots(p1a):
+    """8 slots sharing one paged q8_0 pool, lengths log-uniform in [1024, 32768] (scaled down 8x here; the full size
+    runs in test_full_size_configs), page tables interleaved, one row per slot"""
+    Hq, Hkv, D, psh = 24, 4, 256, 8
+    g = I.rng(33)
+    lens = [int(np.exp(g.uniform(np.log(128), np.log(4096)))) for _ in range(8)]
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, psh, lens, seed=33)
+    q, _, _, gate = I.qkv(34, 1, 8, Hq, Hkv, D)
+    pos = np.array([n - 1 for n in lens], np.int32)
+    rtab = np.array([s * pool.maxp for s in range(8)], np.int32)
+    ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, 1 / 16, gate=gate)
+    out = torch.empty((8, Hq, D), device="cuda")
+    p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, 8, dev(pos), Hq, 1 / 16, gate=dev(gate))
+    check(out.cpu().numpy(), ref, "config 3 (reduced)")
+
+
+@pytest.mark.parametrize("kv_type", [O.KV_Q4_0, O.KV_Q8_0])
+def test_config4_verify_blocks(p1a, kv_type):
+    """MTP verify: 4 sequences x 4 rows (1 accepted + 3 drafts), causal inside the block, f16-rounded inputs; context
+    reduced to 4096 here"""
+    Hq, Hkv, D, psh, n = 24, 4, 256, 8, 4096
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n] * 4, seed=44, f16_inputs=True)
+    q, _, _, _ = I.qkv(45, 1, 16, Hq, Hkv, D, f16_inputs=True)
+    pos = np.array([n - 4 + t for _ in range(4) for t in range(4)], np.int32)
+    rtab = np.array([s * pool.maxp for s in range(4) for _ in range(4)], np.int32)
+    ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, 1 / 16)
+    out = torch.empty((16, Hq, D), device="cuda")
+    p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, 16, dev(pos), Hq, 1 / 16, rows_per_seq=4)
+    check(out.cpu().numpy(), ref, "config 4 (reduced)")
+
+
+def test_other_shapes_and_refusals(p1a):
+    # GQA 4 / D 128 f16, GQA 8 / D 64 f16 (MFMA path), q8_0 at D 128 (generic path)
+    for kv_type, Hq, Hkv, D in [(O.KV_F16, 8, 2, 128), (O.KV_F16, 8, 1, 64), (O.KV_Q8_0, 8, 2, 128), (O.KV_Q4_0, 6, 3, 96)]:
+        pool = Pool(p1a, kv_type, Hq, Hkv, D, 6, [333], seed=D)
+        q, _, _, gate = I.qkv(D + 1, 1, 2, Hq, Hkv, D)
+        ref = O.attn_rows(pool.host_seq(0), q, np.array([330, 331], np.int32), Hq, 0.1, gate=gate)
+        out = run_decode(p1a, pool.dev_seq(0), q, 2, 330, Hq, 0.1, gate=gate)
+        check(out, ref, f"shape {kv_type} {Hq}/{Hkv}/{D}")
+    pool = Pool(p1a, O.KV_F16, 4, 2, 64, 4, [64], seed=1)
+    out = torch.full((1, 5, 64), 7.0, device="cuda")
+    with pytest.raises(p1a.P1AError):
+        p1a.attn_decode(out, pool.dev_seq(0), out, 1, 5, 5, 0.125)      # Hq not a multiple of Hkv
+    torch.cuda.synchronize()
+    assert torch.all(out == 7.0)                                        # refused: out untouched
