@@ -1,0 +1,83 @@
+"""Chunked causal prefill on the GPU (through the C ABI) vs the CPU oracle: append the chunk (codes bit-exact), then
+attention with the fused gate. Tolerance of the path: max-abs 2e-3, rel-L2 1e-3 vs the fp32 oracle."""
+import numpy as np
+import pytest
+import torch
+
+import _inputs as I
+import _oracle as O
+from _gpu import Pool, check, dev
+
+pytestmark = pytest.mark.gpu
+TYPES = [O.KV_F16, O.KV_Q8_0, O.KV_Q4_0]
+
+
+def run_prefill(p1a, c, q, T, p0, Hq, scale, gate=None):
+    out = torch.full((T, Hq, c.D), float("nan"), device="cuda")
+    p1a.attn_prefill(dev(q), c, out, T, p0, Hq, scale, gate=None if gate is None else dev(gate))
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("p0,T", [(0, 1), (0, 200), (37, 100), (300, 129), (1000, 260)])
+def test_prefill_vs_oracle(p1a, kv_type, p0, T):
+    Hq, Hkv, D, psh = 12, 2, 256, 5
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [p0 + T, 50], seed=7 + p0, n_layers=2, layer=1)
+    q, _, _, gate = I.qkv(500 + T, 1, T, Hq, Hkv, D, f16_inputs=True)
+    pos = p0 + np.arange(T, dtype=np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, 1 / 16, gate=gate)
+    out = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16, gate=gate)
+    check(out, ref, f"prefill type {kv_type} p0 {p0} T {T}")
+
+
+@pytest.mark.parametrize("kv_type,Hq,Hkv,D,psh", [(O.KV_F16, 4, 1, 64, 4), (O.KV_Q8_0, 8, 2, 128, 6), (O.KV_Q4_0, 4, 2, 64, 8), (O.KV_F16, 6, 1, 128, 7)])
+def test_other_shapes(p1a, kv_type, Hq, Hkv, D, psh):
+    p0, T = 100, 150
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [p0 + T], seed=D + psh)
+    q, _, _, _ = I.qkv(D, 1, T, Hq, Hkv, D)
+    pos = p0 + np.arange(T, dtype=np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, 0.1)
+    out = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 0.1)
+    check(out, ref, f"prefill shape {kv_type} {Hq}/{Hkv}/{D} psh {psh}")
+    # contiguous cache gives the same bits as the paged one
+    out2 = run_prefill(p1a, pool.dev_contiguous(0), q, T, p0, Hq, 0.1)
+    assert np.array_equal(out, out2)
+
+
+def test_config5_append_then_prefill_reduced(p1a):
+    """config 5 at 1/8 scale: 3584 tokens already in q8_0 pages, a 512-token chunk is quantized on append (codes
+    bit-exact vs the oracle), then causal attention with the fused gate"""
+    Hq, Hkv, D, psh, p0, T = 24, 4, 256, 8, 3584, 512
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, psh, [p0 + T], seed=55, f16_inputs=False, fill="none")
+    k, v = pool.k[0], pool.v[0]
+    O.kv_append_rows(pool.host_seq(0), k, v, np.arange(p0 + T))
+    c = pool.dev_seq(0)
+    p1a.kv_append(c, dev(k[:p0]), dev(v[:p0]), 0, p0)           # history
+    p1a.kv_append(c, dev(k[p0:]), dev(v[p0:]), p0, T)           # the chunk's own K/V, before attention
+    torch.cuda.synchronize()
+    assert np.array_equal(pool.dpool.cpu().numpy(), pool.host.pool)
+    q, _, _, gate = I.qkv(56, 1, T, Hq, Hkv, D, f16_inputs=True)
+    rows = np.array([0, 1, 127, 128, 255, 300, 511])               # oracle on a sample of the rows
+    ref = O.attn_rows(pool.host_seq(0), q[rows], (p0 + rows).astype(np.int32), Hq, 1 / 16, gate=gate[rows])
+    out = run_prefill(p1a, c, q, T, p0, Hq, 1 / 16, gate=gate)
+    assert np.all(np.isfinite(out))
+    check(out[rows], ref, "config 5 (reduced)")
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_prefill_rows_match_decode(p1a, kv_type):
+    """mirror of the reference's prefill-vs-decode test: every prefill row is the decode result at its position
+    (both paths round Q, K, V and P to f16 once, so they agree far inside the tolerance)"""
+    Hq, Hkv, D, psh, p0, T = 12, 2, 256, 8, 700, 140
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [p0 + T], seed=91)
+    q, _, _, _ = I.qkv(92, 1, T, Hq, Hkv, D)
+    out = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16)
+    dq = dev(q)
+    dec = torch.empty((T, Hq, D), device="cuda")
+    for t0 in range(0, T, 4):
+        n = min(4, T - t0)
+        p1a.attn_decode(dq[t0:t0 + n], pool.dev_seq(0), dec[t0:t0 + n], n, p0 + t0, Hq, 1 / 16)
+    torch.cuda.synchronize()
+    ma, rl = I.errors(out, dec.cpu().numpy())
+    assert ma < 1e-3 and rl < 5e-4, (ma, rl)
