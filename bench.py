@@ -26,9 +26,9 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
-def build_pool(p1a, torch, kv_type, Hq, Hkv, D, psh, n_ctx, n_seq, seed):
-    """n_seq sequences of n_ctx tokens in one paged pool, page tables a random permutation; K/V are N(0,1), K
-    RMS-normed per head, written through the library's own quantize-on-append."""
+def build_pool(p1a, torch, kv_type, Hq, Hkv, D, psh, n_ctx, n_seq, seed, lens=None):
+    """n_seq sequences of n_ctx tokens (or lens[s]) in one paged pool, page tables a random permutation; K/V are
+    N(0,1), K RMS-normed per head, written through the library's own quantize-on-append."""
     ps = 1 << psh
     ppseq = (n_ctx + ps - 1) // ps
     n_pages = ppseq * n_seq
@@ -39,8 +39,9 @@ def build_pool(p1a, torch, kv_type, Hq, Hkv, D, psh, n_ctx, n_seq, seed):
     chunk = 4096
     for s in range(n_seq):
         c = kv.slot(s, ppseq)
-        for a in range(0, n_ctx, chunk):
-            T = min(chunk, n_ctx - a)
+        n_s = n_ctx if lens is None else lens[s]
+        for a in range(0, n_s, chunk):
+            T = min(chunk, n_s - a)
             k = torch.randn((T, Hkv, D), generator=g, device="cuda")
             k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + 1e-6)
             v = torch.randn((T, Hkv, D), generator=g, device="cuda")
@@ -71,6 +72,81 @@ def time_graph(torch, stream, fn_list, warmup):
         e1.synchronize()
         torch.cuda.synchronize()
     return e0.elapsed_time(e1) * 1e-3 / len(fn_list)
+
+
+def time_eager(torch, fn, reps, warmup=2):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) * 1e-3 / reps
+
+
+def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
+    """secondary measurements: the other BASELINE.json configs at full size (reported, not the headline value)"""
+    import math
+    ex = {}
+    g = torch.Generator(device="cuda").manual_seed(5)
+
+    def normed(shape):
+        x = torch.randn(shape, generator=g, device="cuda")
+        return x * torch.rsqrt((x * x).mean(-1, keepdim=True) + 1e-6)
+
+    # configs[4]: chunked prefill, T = 4096 after 28672 tokens, q8_0, append of the chunk then attention + gate
+    p0, T = 28672, 4096
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, p0 + T, 1, seed=21)
+    c = kv.slot(0, ppseq)
+    q = normed((T, Hq, D)).half().float()
+    gate = torch.randn((T, Hq * D), generator=g, device="cuda")
+    out = torch.empty((T, Hq, D), device="cuda")
+    kc = normed((T, Hkv, D))
+    vc = torch.randn((T, Hkv, D), generator=g, device="cuda")
+    sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=5)
+    flop = 4.0 * D * Hq * (p0 * T + T * (T + 1) / 2)
+    ex["prefill_T4096_p28672_q8_0_ms"] = round(sec * 1e3, 4)
+    ex["prefill_TFLOPs"] = round(flop / sec / 1e12, 1)
+    ex["prefill_frac_of_f16_mfma_peak"] = round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)
+    sec = time_eager(torch, lambda: p1a.kv_append(c, kc, vc, p0, T), reps=20)
+    ab = 2 * T * Hkv * D * 4 + 2 * T * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
+    ex["append_T4096_q8_0_us"] = round(sec * 1e6, 2)
+    ex["append_GBs"] = round(ab / sec / 1e9, 1)
+    del kv, c, q, gate, out
+    # configs[3]: MTP verify, 4 sequences x 4 rows, q4_0, ctx 65536
+    n4 = 65536
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q4_0, Hq, Hkv, D, psh, n4, 4, seed=22)
+    pos = torch.tensor([n4 - 4 + t for _ in range(4) for t in range(4)], dtype=torch.int32, device="cuda")
+    rt = torch.tensor([s * ppseq for s in range(4) for _ in range(4)], dtype=torch.int32, device="cuda")
+    q = normed((16, Hq, D)).half().float()
+    out = torch.empty((16, Hq, D), device="cuda")
+    cr = kv.with_rows(rt)
+    with torch.cuda.stream(stream):
+        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 16, pos, Hq, scale, rows_per_seq=4)] * 20, 2)
+    vb = 4 * n4 * 2 * p1a.kv_row_bytes(p1a.KV_Q4_0, Hkv, D)
+    ex["verify_4x4_q4_0_64K_us"] = round(sec * 1e6, 2)
+    ex["verify_GBs"] = round(vb / sec / 1e9, 1)
+    del kv, cr
+    # configs[2]: 8 slots, one row each, ctx log-uniform in [1024, 32768], q8_0, one shared pool
+    rs = torch.Generator().manual_seed(8)
+    lens = [int(math.exp(float(torch.empty(1).uniform_(math.log(1024), math.log(32768), generator=rs)))) for _ in range(8)]
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, 32768, 8, seed=23, lens=lens)
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32, device="cuda")
+    rt = torch.tensor([s * ppseq for s in range(8)], dtype=torch.int32, device="cuda")
+    q = normed((8, Hq, D))
+    gate = torch.randn((8, Hq * D), generator=g, device="cuda")
+    out = torch.empty((8, Hq, D), device="cuda")
+    cr = kv.with_rows(rt)
+    with torch.cuda.stream(stream):
+        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 8, pos, Hq, scale, gate=gate)] * 20, 2)
+    bb = sum(lens) * 2 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
+    ex["batched_8slots_q8_0_us"] = round(sec * 1e6, 2)
+    ex["batched_GBs"] = round(bb / sec / 1e9, 1)
+    ex["batched_ctx"] = lens
+    return ex
 
 
 def cpu_baseline(Hq, Hkv, D, n_ctx, seed):
@@ -149,6 +225,8 @@ def main():
         "extra": {"same_pool_GBs": round(step_bytes / sec_same / 1e9, 1), "same_pool_us": round(sec_same * 1e6, 2),
                   "nsplit": p1a.get_nsplit(Hkv)},
     }
+    if not args.no_extra:
+        res["extra"].update(extras(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     if not args.no_cpu:
         cb, ref, (hq, hgate, hc) = cpu_baseline(Hq, Hkv, D, n_ctx, seed=7)
         res["cpu_baseline"] = cb

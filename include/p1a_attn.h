@@ -120,6 +120,9 @@ int p1a_warmup(int rows, int Hq, int Hkv, int D, void *stream);
  * attn_dec2_nsplit / attn_dec2_set_nsplit, src/fast/attn_dec2.cuh:19-20. Never change it between graph captures. */
 int p1a_get_nsplit(int Hkv);
 void p1a_set_nsplit(int n);
+/* Benchmarks only (no counterpart in the reference, whose benches time both kernels together): when on,
+ * p1a_attn_decode stops after the split-K kernel and leaves `out` untouched, so that kernel can be event-timed alone. */
+void p1a_bench_skip_merge(int on);
 /* free every scratch buffer of the current process (after synchronising the devices that own them) */
 void p1a_release(void);
 

@@ -8,7 +8,8 @@ KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
     "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_decode", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
-    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_release", "p1a_last_error", "p1a_version",
+    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_release", "p1a_last_error",
+    "p1a_version",
 ]
 
 
@@ -60,6 +61,8 @@ def lib():
     L.p1a_get_nsplit.argtypes = [i32]
     L.p1a_set_nsplit.restype = None
     L.p1a_set_nsplit.argtypes = [i32]
+    L.p1a_bench_skip_merge.restype = None
+    L.p1a_bench_skip_merge.argtypes = [i32]
     L.p1a_release.restype = None
     L.p1a_last_error.restype = ctypes.c_char_p
     L.p1a_version.restype = ctypes.c_char_p
@@ -199,3 +202,7 @@ def get_nsplit(Hkv):
 
 def set_nsplit(n):
     lib().p1a_set_nsplit(n)
+
+
+def bench_skip_merge(on):
+    lib().p1a_bench_skip_merge(1 if on else 0)

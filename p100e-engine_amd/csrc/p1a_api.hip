@@ -30,6 +30,7 @@ scratch g_scr[MAX_SCR];
 int g_nscr = 0;
 std::mutex g_mu;
 int g_nsplit_override = 0;
+bool g_skip_merge = false;
 int g_cus[16] = {0};
 
 int cu_count() {
@@ -126,6 +127,7 @@ int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float 
     while (pos_rows && rows_per_seq > 1 && rows_per_seq % a.rows_per_group) --a.rows_per_group;
     a.nsplit = nsplit_req();
     a.cus = cu_count();
+    a.skip_merge = g_skip_merge;
     size_t need_o, need_ml;
     decode_scratch_need(*c, Hq, T < 8 ? 8 : T, a.rows_per_group, a.nsplit, a.cus, need_o, need_ml);
     scratch * sc = scratch_for(s, need_o, need_ml);
@@ -176,6 +178,8 @@ int p1a_get_nsplit(int Hkv) {
 }
 
 void p1a_set_nsplit(int n) { g_nsplit_override = n > 0 ? n : 0; }
+
+void p1a_bench_skip_merge(int on) { g_skip_merge = on != 0; }
 
 void p1a_release(void) {
     std::lock_guard<std::mutex> lk(g_mu);

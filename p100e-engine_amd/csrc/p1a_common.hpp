@@ -60,6 +60,7 @@ struct decode_args {
     float scale;
     int nsplit;           // requested split streams (0 = default for the device)
     int cus;              // compute units of the device
+    bool skip_merge;      // benchmarks only: stop after the split-K kernel
     float * part_o;       // [T*Hq][nsplit][D]
     float * part_ml;      // [T*Hq][nsplit][2]
 };

@@ -1,22 +1,28 @@
 // Split-K paged-KV decode / MTP-verify attention for gfx950 (MI355X).
 //
 // Work decomposition
-//   grid = (nsplit, Hkv / HPW, row groups), block = 4 waves. A row group is up to 4 query rows of ONE sequence (the
-//   tokens of a verify block); its GQA * rows query rows are the columns of 16-wide MFMA tiles, so the group's KV is
-//   read once. Wave w owns kv head (w % HPW) and key sub-tile (w / HPW): it walks 32-key tiles of that head, the
-//   tiles of split stream s being the units s, s + nsplit, ... of 32 * (4 / HPW) positions. The partition depends
-//   only on the device and Hkv, never on T, the depth or the batch, so every row is computed by the same sequence of
-//   operations whichever call it is part of (T-invariance, rows == single, paged == contiguous).
-//   A wave's tile (32 keys x one head, K and V) is fetched with 16-byte loads in memory order (17 consecutive lanes
-//   cover one q8_0 head row), parked in a wave-private LDS tile and read back in MFMA operand order; no workgroup
-//   barrier is needed inside the key loop.
+//   grid = (nsplit * head groups, row groups), block = NW waves (8, or 4 when a tile is large). A row group is up to
+//   4 query rows of ONE sequence (the tokens of a verify block); its GQA * rows query rows are the columns of 16-wide
+//   MFMA tiles, so the group's KV is read once. Wave w owns kv head (w % HPW) of the workgroup's head group and key
+//   sub-range (w / HPW): in unit u (32 * NW / HPW positions) it owns 32 consecutive positions, which it walks as two
+//   16-key tiles; split stream s owns the units s, s + nsplit, ... . The partition depends only on the device and
+//   Hkv, never on T, the depth or the batch, so a row is computed by the same sequence of operations whichever call
+//   it is part of (T-invariance, rows == single, paged == contiguous).
+// Data movement
+//   A 16-key tile of one head (K or V) is fetched by global_load_lds_dwordx4: 16 bytes per lane in memory order (17
+//   consecutive lanes cover one q8_0 head row), written by the memory pipeline straight into a wave-private LDS slot
+//   that is the linear image of those rows - no staging registers, no workgroup barrier in the key loop. K and V have
+//   two slots each; the tile two steps ahead is requested as soon as a slot has been consumed, so every wave keeps
+//   about three tiles in flight while it computes. Each slot is its own __shared__ array so that the compiler can
+//   tell which outstanding load a given LDS read depends on and wait for exactly that one.
 // Arithmetic
-//   S^T = K Q^T and O^T = V^T P^T on v_mfma_f32_16x16x32_f16: q8_0 codes are expanded to f16 in registers with a
-//   byte-permute (0x6400 | code ^ 0x80 = 1152 + code) and multiplied by the f16 block scale; V is read from LDS with
-//   the transposing ds_read_b64_tr_b8 / _tr_b16 so that a lane holds 8 keys of one output dim. Q is pre-multiplied by
-//   scale * log2(e) and rounded to f16, P = 2^(S - m) is rounded to f16, all accumulation is fp32. The softmax
-//   denominator is one more MFMA against an all-ones operand, so it sums exactly the P that multiplies V.
-//   Partials (m, l, O) go to scratch and merge_k folds them in split order and applies the sigmoid gate.
+//   S^T = K Q^T on v_mfma_f32_16x16x32_f16 and O^T = V^T P^T on v_mfma_f32_16x16x16_f16: q8_0 codes are expanded to
+//   f16 in registers with a byte-permute (0x6400 | code ^ 0x80 = 1152 + code) and multiplied by the f16 block scale;
+//   V is read from LDS with the transposing ds_read_b64_tr_b8 / _tr_b16 so that a lane holds 4 keys of one output
+//   dim. Q is pre-multiplied by scale * log2(e) and rounded to f16, P = 2^(S - m) is rounded to f16, all accumulation
+//   is fp32. The softmax denominator is one more MFMA against an all-ones operand, so it sums exactly the P that
+//   multiplies V. The waves of one head fold their (m, l, O) through LDS; one partial per (workgroup, head) goes to
+//   scratch and merge_k folds the splits in a fixed order and applies the sigmoid gate.
 #include "p1a_common.hpp"
 
 #include <cstdlib>
@@ -29,15 +35,14 @@ constexpr float NEG_INF = -__builtin_inff();
 template <uint32_t KT, int D> struct tile_cfg {
     static constexpr int HB = (int) head_bytes(KT, D);
     static constexpr int CPK = HB / 16;                        // 16-byte chunks per (key, head)
-    static constexpr int KSTR = (CPK & 1) ? HB : HB + 16;      // LDS row stride: an odd number of 16-byte units
-    static constexpr int NCH = 32 * CPK;                       // chunks per 32-key tile
+    static constexpr int NCH = 16 * CPK;                       // chunks per 16-key tile
     static constexpr int NRND = (NCH + 63) / 64;               // load rounds per tile
-    static constexpr int TILE_B = 32 * KSTR;
-    static constexpr int TAB_B = KT == P1A_KV_F16 ? 0 : (D / 32) * 64;   // transposed V scale table
-    static constexpr int WAVE_B = 2 * TILE_B + TAB_B;
-    static constexpr int NMF = D / 32;                         // QK MFMAs per 16-key sub-tile
+    static constexpr int SLOT_B = 16 * HB;                     // one LDS slot: the linear image of 16 head rows
+    static constexpr int TAB_B = 256;                          // per wave: transposed V scales, later (m, l) of the merge
+    static constexpr int NMF = D / 32;                         // QK MFMAs per tile
     static constexpr int NDT = D / 16;                         // output dim tiles
     static_assert(HB % 16 == 0, "head row must be a whole number of 16-byte chunks");
+    static_assert(SLOT_B >= 16 * (D / 4) * 4, "a slot must hold one dim quarter of a wave's accumulators");
 };
 
 #ifdef P1A_TRACE
@@ -60,21 +65,10 @@ struct dec_params {
     const int32_t * pos_rows;
     int T, RG, Hq, Hkv, GQA, HPW;
     float qscale;     // softmax scale * log2(e)
-    int nsplit;       // split streams (grid.x)
+    int nsplit;       // split streams
 };
 
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
-
-// 4 int8 codes (one dword) -> 4 halves holding 1152 + code, as two packed pairs
-__device__ __forceinline__ void codes4_to_h(uint32_t w, h2 & a, h2 & b) {
-    const uint32_t x = w ^ 0x80808080u;
-    a = __builtin_bit_cast(h2, perm(0x64646464u, x, 0x04010400u));
-    b = __builtin_bit_cast(h2, perm(0x64646464u, x, 0x04030402u));
-}
-
-// 16-byte global load that the compiler cannot turn into something narrower
-__device__ __forceinline__ i4 ldg16(const char * p) { return *reinterpret_cast<const i4 *>(p); }
-
 __device__ __forceinline__ int rfl(int x) { return __builtin_amdgcn_readfirstlane(x); }
 __device__ __forceinline__ size_t rfl64(size_t x) {
     const uint32_t lo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) x);
@@ -82,19 +76,53 @@ __device__ __forceinline__ size_t rfl64(size_t x) {
     return ((size_t) hi << 32) | lo;
 }
 
-// 4 int8 codes -> (code * d) as two packed f16 pairs, returned as raw dwords so that MFMA operands are built in place
+// 4 int8 codes (one dword) -> (code * d) as two packed f16 pairs, returned as raw dwords so MFMA operands are built in place
 struct u2 { uint32_t lo, hi; };
 __device__ __forceinline__ u2 deq4(uint32_t w, h2 d01, h2 d23) {
     const h2 off = {(half_t) 1152, (half_t) 1152};
-    h2 a, b;
-    codes4_to_h(w, a, b);
+    const uint32_t x = w ^ 0x80808080u;
+    const h2 a = __builtin_bit_cast(h2, perm(0x64646464u, x, 0x04010400u));
+    const h2 b = __builtin_bit_cast(h2, perm(0x64646464u, x, 0x04030402u));
     return u2{__builtin_bit_cast(uint32_t, (a - off) * d01), __builtin_bit_cast(uint32_t, (b - off) * d23)};
 }
+
+// ---- hand-issued memory operations of the tile ring ----
+// The tile loads are global_load_lds_dwordx4 (global -> LDS, 16 bytes per lane, lane i lands at M0 + 16 i). They are
+// written as inline assembly so that the waits on them can be partial: the vector-memory counter retires in order,
+// so "at most n newer loads outstanding" (s_waitcnt vmcnt(n)) is exactly "tile x has landed" when every tile is NR
+// loads. For the same reason nothing else in the key loop may be a vector load: the page-table entry of a tile is
+// fetched with a scalar load, issued one step ahead.
+__device__ __forceinline__ uint32_t lds_addr(const char * p) { return (uint32_t) (size_t) (const __attribute__((address_space(3))) char *) p; }
+__device__ __forceinline__ void dma16(const char * sbase, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+}
+__device__ __forceinline__ void dma16v(const char * vaddr, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(vaddr), "s"(lds) : "memory", "m0");
+}
+template <int N> __device__ __forceinline__ void wait_vm_imm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
+// wait until at most `newer` tile fetches (NR loads each) issued after the wanted one are still in flight
+template <int NR> __device__ __forceinline__ void wait_tiles(int newer) {
+    if (newer <= 0) wait_vm_imm<0>();
+    else if (newer == 1) wait_vm_imm<NR>();
+    else if (newer == 2) wait_vm_imm<2 * NR>();
+    else wait_vm_imm<3 * NR>();
+}
+__device__ __forceinline__ int sload_i32(const int32_t * p) {
+    int v;
+    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(v) : "s"(p));
+    return v;
+}
+__device__ __forceinline__ void wait_scalar(int & v) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(v)); }
 
 template <uint32_t KT, int D, int NT, int NWV>
 __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
-    __shared__ __attribute__((aligned(16))) char lds[NWV * C::WAVE_B];
+    // four tile slots per wave (K and V, two each) as separate arrays, plus a small per-wave table
+    __shared__ __attribute__((aligned(16))) char kb0[NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char kb1[NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char vb0[NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char vb1[NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char tabs[NWV * C::TAB_B];
 
     const int lane = threadIdx.x & 63, wave = rfl(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
@@ -118,20 +146,22 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     const int nr = min(P.RG, P.T - row0);                     // rows of this group
     const int R = nr * P.GQA;                                 // live MFMA columns
     const int p0v = P.pos_rows ? 0 : (P.p0_dev ? *P.p0_dev : P.p0);
-
     TS(0);
-    char * kt = lds + wave * C::WAVE_B;
-    char * vt = kt + C::TILE_B;
-    char * tab = vt + C::TILE_B;
+
+    char * const ks0 = kb0 + wave * C::SLOT_B, * const ks1 = kb1 + wave * C::SLOT_B;
+    char * const vs0 = vb0 + wave * C::SLOT_B, * const vs1 = vb1 + wave * C::SLOT_B;
+    char * const tab = tabs + wave * C::TAB_B;
 
     // visible-position limit of each of this lane's columns, and the group's maximum
     int plim[NT];
-    int n_max = 0;
+    int n_max = 0, p_min = 0x7fffffff;
     for (int t = 0; t < nr; ++t) {
         const int pt_ = P.pos_rows ? P.pos_rows[row0 + t] : p0v + row0 + t;
         n_max = max(n_max, pt_ + 1);
+        p_min = min(p_min, pt_);
     }
     n_max = rfl(n_max);
+    p_min = rfl(p_min);
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         const int col = 16 * r + c;
@@ -144,99 +174,52 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     const int32_t * ptab = kv_tab(P.pg, P.pos_rows ? row0 : 0);
     const size_t head_off = (size_t) hk * C::HB;
     const int rowb = (int) P.pg.rowb;
-    // a 32-key tile lies in one page (or in a contiguous cache): one base per tile, static per-lane offsets
-    const bool onepage = !ptab || P.pg.psh >= 5;
 
-    int lofs[C::NRND], soff[C::NRND];
+    // chunk i = 64 * round + lane of a tile is bytes [16 cir, +16) of key i / CPK; static per-lane source offsets
+    unsigned soff[C::NRND];
 #pragma unroll
     for (int rd = 0; rd < C::NRND; ++rd) {
         const int i = rd * 64 + lane;
         const int key = i / C::CPK, cir = i - key * C::CPK;
-        lofs[rd] = key * C::KSTR + cir * 16;
-        soff[rd] = key * rowb + (int) head_off + cir * 16;
+        soff[rd] = (unsigned) (key * rowb + (int) head_off + cir * 16);
     }
 
-    // 16 bytes per lane in memory order; keys past `last` (beyond every row's visible range) are clamped onto it, so
-    // nothing outside the sequence is ever read
-    auto issue = [&](i4 * regs, const char * base, int ts, int last) {
-        const size_t off0 = rfl64(kv_off_tab(P.pg, ptab, ts));
-        if (onepage && last >= 31) {
-            const char * b0 = base + off0;
-#pragma unroll
-            for (int rd = 0; rd < C::NRND; ++rd)
-                if (C::NCH % 64 == 0 || rd * 64 + lane < C::NCH) regs[rd] = ldg16(b0 + soff[rd]);
-        } else {
-            const size_t off1 = last >= 16 ? rfl64(kv_off_tab(P.pg, ptab, ts + 16)) : off0;
-#pragma unroll
-            for (int rd = 0; rd < C::NRND; ++rd) {
-                const int i = rd * 64 + lane;
-                const int key = i / C::CPK, cir = i - key * C::CPK;
-                const int kcl = min(key, last);
-                const size_t go = ((kcl & 16) ? off1 : off0) + (size_t) ((kcl & 15) * rowb) + head_off + (size_t) (cir * 16);
-                if (C::NCH % 64 == 0 || i < C::NCH) regs[rd] = ldg16(base + go);
-            }
+    // Tile t of this wave (t = 0, 1, ...): unit split + (t >> 1) * nsplit, keys [ts, ts + 16) with
+    // ts = unit * U + sub * 32 + 16 * (t & 1). A 16-key tile never straddles a page (pages hold >= 16 positions).
+    auto tile_start = [&](int t) { return (split + (t >> 1) * P.nsplit) * U + sub * 32 + 16 * (t & 1); };
+    // One of the NR loads of a tile: round rd of the tile at `ts` into `slot`. Keys past the last visible position are
+    // clamped onto it (never weighted), so nothing outside the sequence is read. A tile is always exactly NR loads.
+    auto tile_off = [&](int ts, int page) -> size_t {
+        if (!ptab) return (size_t) ts * P.pg.rowb;
+        return (size_t) page * P.pg.pstride + (size_t) (ts & ((1 << P.pg.psh) - 1)) * P.pg.rowb;
+    };
+    auto fetch_round = [&](char * slot, const char * b0, int ts, int rd) {
+        const int last = n_max - 1 - ts;
+        const int i = rd * 64 + lane;
+        uint32_t off = soff[rd];
+        if (last < 15) {
+            const int key = i / C::CPK, cir = i - key * C::CPK;
+            off = (uint32_t) (min(key, last) * rowb + (int) head_off + cir * 16);
         }
+        if (C::NCH % 64 == 0 || i < C::NCH) dma16(b0, off, lds_addr(slot) + rd * 1024);
     };
-    // the same loads written straight into an LDS tile (global_load_lds_dwordx4: lane i of a round lands at
-    // tile + round * 1024 + 16 i), usable when the tile is the linear image of the head rows (KSTR == HB)
-    auto issue_lds = [&](char * tile, const char * base, int ts, int last) {
-        const size_t off0 = rfl64(kv_off_tab(P.pg, ptab, ts));
-        if (onepage && last >= 31) {
-            const char * b0 = base + off0;
-#pragma unroll
-            for (int rd = 0; rd < C::NRND; ++rd)
-                if (C::NCH % 64 == 0 || rd * 64 + lane < C::NCH)
-                    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *) (b0 + soff[rd]),
-                                                     (void __attribute__((address_space(3))) *) (tile + rd * 1024), 16, 0, 0);
-        } else {
-            const size_t off1 = last >= 16 ? rfl64(kv_off_tab(P.pg, ptab, ts + 16)) : off0;
-#pragma unroll
-            for (int rd = 0; rd < C::NRND; ++rd) {
-                const int i = rd * 64 + lane;
-                const int key = i / C::CPK, cir = i - key * C::CPK;
-                const int kcl = min(key, last);
-                const char * src = base + ((kcl & 16) ? off1 : off0) + (size_t) ((kcl & 15) * rowb) + head_off + (size_t) (cir * 16);
-                if (C::NCH % 64 == 0 || i < C::NCH)
-                    __builtin_amdgcn_global_load_lds((const void __attribute__((address_space(1))) *) src,
-                                                     (void __attribute__((address_space(3))) *) (tile + rd * 1024), 16, 0, 0);
-            }
-        }
-    };
-    auto park = [&](char * tile, const i4 * regs) {
-#pragma unroll
-        for (int rd = 0; rd < C::NRND; ++rd)
-            if (C::NCH % 64 == 0 || rd * 64 + lane < C::NCH) *reinterpret_cast<i4 *>(tile + lofs[rd]) = regs[rd];
-    };
+    auto page_of = [&](int ts) -> const int32_t * { return ptab + (ts >> P.pg.psh); };
 
-    f4 o[NT][C::NDT];
-    f4 ol[NT];
-    float m_run[NT];
+    // first requests: K then V of tile 0; every later tile is requested, one load at a time, from inside the step
+    // before it, so that a wave is never parked on the memory pipeline for long while it has products to compute
+    const bool have0 = tile_start(0) < n_max;
+    if (have0) {
+        int pg0 = 0;
+        if (ptab) pg0 = sload_i32(page_of(tile_start(0)));
+        wait_scalar(pg0);
+        const size_t o0 = tile_off(tile_start(0), pg0);
 #pragma unroll
-    for (int r = 0; r < NT; ++r) {
-        m_run[r] = NEG_INF;
-        ol[r] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ks0, P.kc + o0, tile_start(0), rd);
 #pragma unroll
-        for (int j = 0; j < C::NDT; ++j) o[r][j] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vs0, P.vc + o0, tile_start(0), rd);
     }
-    const h8 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
+    TS(1);
 
-    // software pipeline: the loads of tile n + 1 are issued into the registers tile n has just vacated
-    constexpr bool KDMA = C::KSTR == C::HB;   // K tiles go global -> LDS directly, V tiles through registers
-    i4 kr[KDMA ? 1 : C::NRND], vr[C::NRND];
-    int u = split;
-    bool have = u * U + sub * 32 < n_max;
-    TS(15);
-    if (have) {
-        const int ts = u * U + sub * 32;
-#ifdef P1A_TRACE
-        { const size_t o_ = rfl64(kv_off_tab(P.pg, ptab, ts)); if (o_ == 1) return; TS(9); }
-#endif
-        if constexpr (KDMA) issue_lds(kt, P.kc, ts, n_max - 1 - ts);
-        else issue(kr, P.kc, ts, n_max - 1 - ts);
-        TS(10);
-        issue(vr, P.vc, ts, n_max - 1 - ts);
-    }
-    TS(14);
     // Q^T operands: column = query row (token t, head hh of the group), 8 consecutive dims per MFMA slot group
     h8 qf[NT][C::NMF];
 #pragma unroll
@@ -249,81 +232,95 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         for (int m = 0; m < C::NMF; ++m) {
             const int d0 = KT == P1A_KV_F16 ? 32 * m + 8 * g : 16 * (4 * (m >> 1) + g) + 8 * (m & 1);
             float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+#ifndef P1A_EXP_NOQ
             if (livec) { a = *reinterpret_cast<const float4 *>(qr + d0); b = *reinterpret_cast<const float4 *>(qr + d0 + 4); }
+#else
+            a.x = (float) (size_t) qr;
+#endif
             const float s = P.qscale;
             qf[r][m] = h8{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s),
                           (half_t) (b.x * s), (half_t) (b.y * s), (half_t) (b.z * s), (half_t) (b.w * s)};
         }
     }
 
-    TS(1);
-    int it_ = 0;
-    while (have) {
-        const int ts = u * U + sub * 32;                      // first position of this wave's tile
-        const int un = u + P.nsplit;
-        const int tsn = un * U + sub * 32;
-        const bool have_n = tsn < n_max;
+    f4 o[NT][C::NDT];
+    f4 ol[NT];
+    float m_run[NT];
+#pragma unroll
+    for (int r = 0; r < NT; ++r) {
+        m_run[r] = NEG_INF;
+        ol[r] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < C::NDT; ++j) o[r][j] = f4{0.f, 0.f, 0.f, 0.f};
+    }
+    const h4 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
 
-        if constexpr (!KDMA) {
-            park(kt, kr);
-            if (have_n) issue(kr, P.kc, tsn, n_max - 1 - tsn);
-        }
-
-        // ---- S^T = K Q^T for the two 16-key sub-tiles ----
-        if (it_ < 1) TS(2 + 5 * it_);
-        f4 s[NT][2];
+    // one 16-key tile from slots (ks, vs); the loads of tile t + 1 into (ksn, vsn) are issued between its products
+    auto step = [&](char * ks, char * vs, char * ksn, char * vsn, int t) {
+        const int ts = tile_start(t);
+        const int tn = tile_start(t + 1);
+        const bool have_n = tn < n_max;
+        int pgn = 0;
+        if (ptab && have_n) pgn = sload_i32(page_of(tn));
+        wait_vm_imm<C::NRND>();                               // K of tile t has landed (only its V is younger)
+        wait_scalar(pgn);
+        const size_t on = have_n ? tile_off(tn, pgn) : 0;
+        const char * const kn = P.kc + on, * const vn = P.vc + on;
+        // ---- S^T = K Q^T ----
+        f4 s[NT];
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
+        for (int r = 0; r < NT; ++r) s[r] = f4{0.f, 0.f, 0.f, 0.f};
+        const char * krow = ks + c * C::HB;
+#ifdef P1A_EXP_NOQK
+        s[0][0] = *reinterpret_cast<const float *>(krow);
+        if (false)
+#endif
+        if constexpr (KT == P1A_KV_F16) {
 #pragma unroll
-            for (int r = 0; r < NT; ++r) s[r][st] = f4{0.f, 0.f, 0.f, 0.f};
-            const char * krow = kt + (16 * st + c) * C::KSTR;
-            if constexpr (KT == P1A_KV_F16) {
+            for (int m = 0; m < C::NMF; ++m) {
+                const h8 a = *reinterpret_cast<const h8 *>(krow + (4 * m + g) * 16);
 #pragma unroll
-                for (int m = 0; m < C::NMF; ++m) {
-                    const h8 a = *reinterpret_cast<const h8 *>(krow + (4 * m + g) * 16);
+                for (int r = 0; r < NT; ++r) s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[r][m], s[r], 0, 0, 0);
+                if (have_n && m < C::NRND) fetch_round(ksn, kn, tn, m);
+            }
+        } else {   // q8_0: 16 B of scales, then 16 chunks of 16 codes
+            const i4 sc = *reinterpret_cast<const i4 *>(krow);
 #pragma unroll
-                    for (int r = 0; r < NT; ++r) s[r][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[r][m], s[r][st], 0, 0, 0);
+            for (int jj = 0; jj < C::NMF / 2; ++jj) {
+                const i4 w = *reinterpret_cast<const i4 *>(krow + 16 + (4 * jj + g) * 16);
+                const uint32_t sw = (uint32_t) sc[jj];
+                const uint32_t d16 = (g & 2) ? (sw >> 16) : (sw & 0xffffu);
+                const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
+                const u2 x0 = deq4((uint32_t) w[0], dd, dd), x1 = deq4((uint32_t) w[1], dd, dd);
+                const u2 x2 = deq4((uint32_t) w[2], dd, dd), x3 = deq4((uint32_t) w[3], dd, dd);
+                const u4 a0 = {x0.lo, x0.hi, x1.lo, x1.hi}, a1 = {x2.lo, x2.hi, x3.lo, x3.hi};
+#pragma unroll
+                for (int r = 0; r < NT; ++r) {
+                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a0), qf[r][2 * jj], s[r], 0, 0, 0);
+                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a1), qf[r][2 * jj + 1], s[r], 0, 0, 0);
                 }
-            } else {   // q8_0: 16 B of scales, then 16 chunks of 16 codes
-                const i4 sc = *reinterpret_cast<const i4 *>(krow);
-#pragma unroll
-                for (int jj = 0; jj < C::NMF / 2; ++jj) {
-                    const i4 w = *reinterpret_cast<const i4 *>(krow + 16 + (4 * jj + g) * 16);
-                    const uint32_t sw = (uint32_t) sc[jj];
-                    const uint32_t d16 = (g & 2) ? (sw >> 16) : (sw & 0xffffu);
-                    const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
-                    const u2 x0 = deq4((uint32_t) w[0], dd, dd), x1 = deq4((uint32_t) w[1], dd, dd);
-                    const u2 x2 = deq4((uint32_t) w[2], dd, dd), x3 = deq4((uint32_t) w[3], dd, dd);
-                    const u4 a0 = {x0.lo, x0.hi, x1.lo, x1.hi}, a1 = {x2.lo, x2.hi, x3.lo, x3.hi};
-#pragma unroll
-                    for (int r = 0; r < NT; ++r) {
-                        s[r][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a0), qf[r][2 * jj], s[r][st], 0, 0, 0);
-                        s[r][st] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a1), qf[r][2 * jj + 1], s[r][st], 0, 0, 0);
-                    }
-                }
+                if (have_n && jj < C::NRND) fetch_round(ksn, kn, tn, jj);
             }
         }
-
-        if (it_ < 1) TS(3 + 5 * it_);
-        if constexpr (KDMA) {   // the K tile has been consumed: fetch the next one into it
-            if (have_n) issue_lds(kt, P.kc, tsn, n_max - 1 - tsn);
+        if (have_n) {   // the rounds the product loop had no place for
+#pragma unroll
+            for (int rd = (KT == P1A_KV_F16 ? C::NMF : C::NMF / 2); rd < C::NRND; ++rd) fetch_round(ksn, kn, tn, rd);
         }
 
-        // ---- online softmax (log2 domain); column = query row, this lane holds keys 16 st + 4 g + i ----
-        h8 pb[NT];
+        // ---- online softmax (log2 domain); column = query row, this lane holds keys ts + 4 g + i ----
+        h4 pb[NT];
         float alpha[NT];
         bool rescale = false;
+        const bool need_mask = ts + 15 > p_min;               // only the last tiles of a sequence hold hidden keys
 #pragma unroll
         for (int r = 0; r < NT; ++r) {
             float mloc = NEG_INF;
 #pragma unroll
-            for (int st = 0; st < 2; ++st)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int kp = ts + 16 * st + 4 * g + i;
-                    s[r][st][i] = kp <= plim[r] ? s[r][st][i] : NEG_INF;
-                    mloc = fmaxf(mloc, s[r][st][i]);
-                }
+            for (int i = 0; i < 4; ++i) {
+                if (need_mask) s[r][i] = ts + 4 * g + i <= plim[r] ? s[r][i] : NEG_INF;
+                else if (plim[r] < 0) s[r][i] = NEG_INF;
+                mloc = fmaxf(mloc, s[r][i]);
+            }
             mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
             const float mnew = fmaxf(m_run[r], mloc);
@@ -331,12 +328,10 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             // nothing accumulated yet (m = -inf): the accumulators are zero and need no rescale
             alpha[r] = (dead || m_run[r] == NEG_INF) ? 1.0f : __builtin_amdgcn_exp2f(m_run[r] - mnew);
             m_run[r] = mnew;
-            float p[8];
+            float p[4];
 #pragma unroll
-            for (int st = 0; st < 2; ++st)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) p[4 * st + i] = dead ? 0.0f : __builtin_amdgcn_exp2f(s[r][st][i] - mnew);
-            pb[r] = h8{(half_t) p[0], (half_t) p[1], (half_t) p[2], (half_t) p[3], (half_t) p[4], (half_t) p[5], (half_t) p[6], (half_t) p[7]};
+            for (int i = 0; i < 4; ++i) p[i] = dead ? 0.0f : __builtin_amdgcn_exp2f(s[r][i] - mnew);
+            pb[r] = h4{(half_t) p[0], (half_t) p[1], (half_t) p[2], (half_t) p[3]};
             rescale = rescale || alpha[r] != 1.0f;
         }
         if (__any(rescale)) {
@@ -348,102 +343,125 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             }
         }
 
-        // ---- V tile to LDS, next V loads into the vacated registers ----
-        if (it_ < 1) TS(4 + 5 * it_);
-        park(vt, vr);
-        if (it_ < 1) TS(5 + 5 * it_);
-        if (have_n) issue(vr, P.vc, tsn, n_max - 1 - tsn);
-
-        // slot e of lane group g is key 4 g + e (e < 4) or 16 + 4 g + e - 4: the keys this lane's P values belong to
+        if (have_n) wait_vm_imm<C::NRND>(); else wait_vm_imm<0>();   // V of tile t has landed (only K of t + 1 is younger)
+        // ---- O^T += V^T P^T: k-slot i of lane group g is key ts + 4 g + i, the key of this lane's P value i ----
+#ifdef P1A_EXP_NOPV
+        o[0][0][0] += *reinterpret_cast<const float *>(vs + lane * 4);
+        if (false)
+#endif
         if constexpr (KT == P1A_KV_F16) {
             const int kk = c >> 2, jq = c & 3;
-            const char * r0 = vt + (4 * g + kk) * C::KSTR + jq * 8;
-            const char * r1 = vt + (16 + 4 * g + kk) * C::KSTR + jq * 8;
+            const char * vr0 = vs + (4 * g + kk) * C::HB + jq * 8;
 #pragma unroll
             for (int j = 0; j < C::NDT; ++j) {
-                const s4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (r0 + j * 32));
-                const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (r1 + j * 32));
-                const h4 l4 = __builtin_bit_cast(h4, lo), h4_ = __builtin_bit_cast(h4, hi);
-                const h8 a = {l4[0], l4[1], l4[2], l4[3], h4_[0], h4_[1], h4_[2], h4_[3]};
+                const s4 w = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (vr0 + j * 32));
+                const h4 a = __builtin_bit_cast(h4, w);
 #pragma unroll
-                for (int r = 0; r < NT; ++r) o[r][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pb[r], o[r][j], 0, 0, 0);
+                for (int r = 0; r < NT; ++r) o[r][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[r], o[r][j], 0, 0, 0);
+                if (have_n && j < C::NRND) fetch_round(vsn, vn, tn, j);
             }
         } else {
-            {   // transposed scale table tab[b][g][e] (f16): one 16-byte row per (block, lane group)
-                const int key = lane & 31, hf = lane >> 5;
-                const i2 sc = *reinterpret_cast<const i2 *>(vt + key * C::KSTR + 8 * hf);
-                const int st = key >> 4, kk = key & 15;
-                char * dst = tab + (kk >> 2) * 16 + ((kk & 3) + 4 * st) * 2;
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const uint32_t wv = (uint32_t) sc[x >> 1];
-                    *reinterpret_cast<uint16_t *>(dst + (4 * hf + x) * 64) = (uint16_t) ((x & 1) ? (wv >> 16) : wv);
-                }
+            {   // transposed scale table tab[block][key] (f16, 32 B per block)
+                const int key = lane & 15, q2 = lane >> 4;    // this lane moves blocks 2 q2 and 2 q2 + 1 of its key
+                const uint32_t sc = *reinterpret_cast<const uint32_t *>(vs + key * C::HB + 4 * q2);
+                *reinterpret_cast<uint16_t *>(tab + (2 * q2) * 32 + key * 2) = (uint16_t) sc;
+                *reinterpret_cast<uint16_t *>(tab + (2 * q2 + 1) * 32 + key * 2) = (uint16_t) (sc >> 16);
             }
+            // one transposing read returns 8 rows: rows 0-3 = keys 4 g .. 4 g + 3 at dims 16 j .., rows 4-7 = the
+            // same keys at dims 16 (j + 1) ..
             const int kk = c >> 1, jb = c & 1;
-            const int key = kk < 4 ? 4 * g + kk : 16 + 4 * g + (kk - 4);
-            const char * vrow = vt + key * C::KSTR + 16 + 8 * jb;
+            const char * vrow = vs + (4 * g + (kk & 3)) * C::HB + 16 + 16 * (kk >> 2) + 8 * jb;
 #pragma unroll
-            for (int j = 0; j < C::NDT; ++j) {
+            for (int j = 0; j < C::NDT; j += 2) {
                 const i2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) (vrow + j * 16));
-                const h8 dv = *reinterpret_cast<const h8 *>(tab + (j >> 1) * 64 + g * 16);
+                const h4 dv = *reinterpret_cast<const h4 *>(tab + (j >> 1) * 32 + g * 8);
                 const u2 x0 = deq4((uint32_t) w[0], h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
-                const u2 x1 = deq4((uint32_t) w[1], h2{dv[4], dv[5]}, h2{dv[6], dv[7]});
-                const u4 a = {x0.lo, x0.hi, x1.lo, x1.hi};
+                const u2 x1 = deq4((uint32_t) w[1], h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
+                const i2 a0 = {(int) x0.lo, (int) x0.hi}, a1 = {(int) x1.lo, (int) x1.hi};
 #pragma unroll
-                for (int r = 0; r < NT; ++r) o[r][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), pb[r], o[r][j], 0, 0, 0);
+                for (int r = 0; r < NT; ++r) {
+                    o[r][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a0), pb[r], o[r][j], 0, 0, 0);
+                    o[r][j + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a1), pb[r], o[r][j + 1], 0, 0, 0);
+                }
+                if (have_n && j / 2 < C::NRND) fetch_round(vsn, vn, tn, j / 2);
             }
         }
+        static_assert(C::NRND <= (KT == P1A_KV_F16 ? C::NDT : C::NDT / 2), "the PV loop must have room for every V load");
 #pragma unroll
-        for (int r = 0; r < NT; ++r) ol[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ones, pb[r], ol[r], 0, 0, 0);
-        u = un;
-        have = have_n;
-        if (it_ < 1) TS(6 + 5 * it_);
-        ++it_;
+        for (int r = 0; r < NT; ++r) ol[r] = __builtin_amdgcn_mfma_f32_16x16x16f16(ones, pb[r], ol[r], 0, 0, 0);
+    };
+
+    for (int t = 0; tile_start(t) < n_max; t += 2) {
+        step(ks0, vs0, ks1, vs1, t);
+        if (tile_start(t + 1) < n_max) step(ks1, vs1, ks0, vs0, t + 1);
     }
     TS(12);
+#ifdef P1A_EXP_NOEPI
+    if (m_run[0] != 12345.f) return;
+#endif
 
     // ---- fold the WPH waves of each head (in sub order) and write one partial per (workgroup, head); the 16
     // columns of one MFMA tile at a time, so that a column is merged the same way whatever NT is. A wave parks its
-    // state in its own (now idle) tile region, so no barrier is needed before the first write ----
-    float * wreg = reinterpret_cast<float *>(lds + wave * C::WAVE_B);   // [16 m][16 l][16 columns][D]
+    // accumulators in its own (now idle) slots, dim quarter k in slot array k, and (m, l) in its table ----
+    constexpr int QD = D / 4;                                 // dims per quarter
+    char * const st[4] = {kb0, kb1, vb0, vb1};
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         const int Rr = min(16, R - 16 * r);                  // live columns of this tile
         if (r) __syncthreads();
         if (c < Rr) {
 #pragma unroll
-            for (int j = 0; j < C::NDT; ++j) *reinterpret_cast<f4 *>(wreg + 32 + c * D + 16 * j + 4 * g) = o[r][j];
-            if (g == 0) { wreg[c] = m_run[r]; wreg[16 + c] = ol[r][0]; }
+            for (int j = 0; j < C::NDT; ++j) {
+                float * dst = reinterpret_cast<float *>(st[j / (C::NDT / 4)] + wave * C::SLOT_B);
+                *reinterpret_cast<f4 *>(dst + c * QD + 16 * (j % (C::NDT / 4)) + 4 * g) = o[r][j];
+            }
+            if (g == 0) {
+                reinterpret_cast<float *>(tab)[c] = m_run[r];
+                reinterpret_cast<float *>(tab)[16 + c] = ol[r][0];
+            }
         }
         __syncthreads();
         const int items = P.HPW * Rr * (D / 4);
         for (int it = threadIdx.x; it < items; it += NWV * 64) {
             const int d4 = it % (D / 4), rest = it / (D / 4);
             const int cc = rest % Rr, hs = rest / Rr;
+            const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
+            const char * sbase = qtr == 0 ? kb0 : qtr == 1 ? kb1 : qtr == 2 ? vb0 : vb1;
             float M = NEG_INF;
             for (int sb = 0; sb < WPH; ++sb)
-                M = fmaxf(M, reinterpret_cast<const float *>(lds + (hs + sb * P.HPW) * C::WAVE_B)[cc]);
+                M = fmaxf(M, reinterpret_cast<const float *>(tabs + (hs + sb * P.HPW) * C::TAB_B)[cc]);
             f4 acc = {0.f, 0.f, 0.f, 0.f};
             float l = 0.f;
             for (int sb = 0; sb < WPH; ++sb) {
-                const float * wr = reinterpret_cast<const float *>(lds + (hs + sb * P.HPW) * C::WAVE_B);
-                const float ms = wr[cc];
+                const int w = hs + sb * P.HPW;
+                const float * tw = reinterpret_cast<const float *>(tabs + w * C::TAB_B);
+                const float ms = tw[cc];
                 if (ms == NEG_INF) continue;
                 const float f = __builtin_amdgcn_exp2f(ms - M);
-                const f4 a = *reinterpret_cast<const f4 *>(wr + 32 + cc * D + 4 * d4);
+                const f4 a = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * QD + dq);
                 acc += a * f;
-                l += wr[16 + cc] * f;
+                l += tw[16 + cc] * f;
             }
             const int col = 16 * r + cc;
             const int t = col / P.GQA, hh = col - t * P.GQA;
             const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) (hg * P.HPW + hs) * P.GQA + hh;
+#if defined(P1A_EXP_NOSTORE)
+            if (M == 12345.f) *reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4) = acc;
+#elif defined(P1A_EXP_NTSTORE)
+            if (M != NEG_INF) __builtin_nontemporal_store(acc, reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4));
+            if (d4 == 0) {
+                float * pm = P.part_ml + (row * P.nsplit + split) * 2;
+                __builtin_nontemporal_store(M, pm);
+                __builtin_nontemporal_store(l, pm + 1);
+            }
+#else
             if (M != NEG_INF) *reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4) = acc;
             if (d4 == 0) {
                 float * pm = P.part_ml + (row * P.nsplit + split) * 2;
                 pm[0] = M;
                 pm[1] = l;
             }
+#endif
         }
     }
     TS(13);
@@ -547,20 +565,45 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
     const int tid = threadIdx.x, q4 = tid & 7, sl = tid >> 3;
     const int d = blockIdx.y * 32 + q4 * 4;
     const float * ml = part_ml + row * NS * 2;
+    constexpr int CH = 8;                                     // splits of a slice fetched together
     float M = NEG_INF;
     for (int s = tid; s < NS; s += 64) M = fmaxf(M, ml[2 * s]);
+    // the partials do not depend on M: request the first batch before the maximum is reduced
+    f4 a[CH];
+    float ms[CH], ls[CH];
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+        const int s = sl + 8 * k;
+        ms[k] = NEG_INF; ls[k] = 0.f; a[k] = f4{0.f, 0.f, 0.f, 0.f};
+        if (s < NS) {
+            ms[k] = ml[2 * s]; ls[k] = ml[2 * s + 1];
+            a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS + s) * D + d);
+        }
+    }
 #pragma unroll
     for (int w = 32; w > 0; w >>= 1) M = fmaxf(M, __shfl_xor(M, w));
     f4 num = {0.f, 0.f, 0.f, 0.f};
     float den = 0.f;
-    for (int s = sl; s < NS; s += 8) {
-        const float ms = ml[2 * s], ls = ml[2 * s + 1];
-        if (ms == NEG_INF || ls == 0.f) continue;
-        const float f = __builtin_amdgcn_exp2f(ms - M);
-        const f4 a = *reinterpret_cast<const f4 *>(part_o + (row * NS + s) * D + d);
-        den = fmaf(f, ls, den);
-        num[0] = fmaf(f, a[0], num[0]); num[1] = fmaf(f, a[1], num[1]);
-        num[2] = fmaf(f, a[2], num[2]); num[3] = fmaf(f, a[3], num[3]);
+    for (int s0 = sl; s0 < NS; s0 += 8 * CH) {
+        if (s0 != sl) {
+#pragma unroll
+            for (int k = 0; k < CH; ++k) {
+                const int s = s0 + 8 * k;
+                ms[k] = NEG_INF; ls[k] = 0.f;
+                if (s < NS) {
+                    ms[k] = ml[2 * s]; ls[k] = ml[2 * s + 1];
+                    a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS + s) * D + d);
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < CH; ++k) {
+            if (ms[k] == NEG_INF || ls[k] == 0.f) continue;   // empty stream: its accumulator was never written
+            const float f = __builtin_amdgcn_exp2f(ms[k] - M);
+            den = fmaf(f, ls[k], den);
+            num[0] = fmaf(f, a[k][0], num[0]); num[1] = fmaf(f, a[k][1], num[1]);
+            num[2] = fmaf(f, a[k][2], num[2]); num[3] = fmaf(f, a[k][3], num[3]);
+        }
     }
     sacc[sl][q4] = num;
     if (q4 == 0) sden[sl] = den;
@@ -626,8 +669,10 @@ dec_plan make_plan(const p1a_kv & c, int Hq, int rows_per_group, int nsplit_req,
     p.RG = rows_per_group < 1 ? 1 : (rows_per_group > cap ? cap : rows_per_group);
     // tuning knobs (development A/B switches, read once): heads per workgroup and waves per workgroup
     static const int env_hpw = env_int("P1A_DEC_HPW", 0), env_nw = env_int("P1A_DEC_NW", 0);
-    int hpw = c.Hkv % 4 == 0 ? 4 : c.Hkv % 2 == 0 ? 2 : 1;
-    if (env_hpw > 0 && env_hpw <= hpw && hpw % env_hpw == 0) hpw = env_hpw;
+    // one kv head per workgroup: its 8 waves fold into ONE partial, which keeps the split traffic at a few percent
+    // of the KV bytes; the head groups of a split stream are placed on one XCD so shared cache lines meet in its L2
+    int hpw = 1;
+    if (env_hpw > 0 && c.Hkv % env_hpw == 0 && (env_hpw == 1 || env_hpw == 2 || env_hpw == 4)) hpw = env_hpw;
     p.HPW = hpw;
     const bool big_tiles = c.type == P1A_KV_F16 && c.D == 256;   // 34 KB of LDS per wave
     p.NW = big_tiles ? 4 : 8;
@@ -706,7 +751,7 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
         else dec_generic_k<P1A_KV_Q4_0><<<grid, 256, 0, s>>>(P);
         rc = hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
     }
-    if (rc != P1A_OK) return rc;
+    if (rc != P1A_OK || a.skip_merge) return rc;
     merge_k<<<dim3(a.T * a.Hq, c.D / 32), 64, 0, s>>>(a.part_o, a.part_ml, a.out, a.gate, pl.NS, c.D);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
