@@ -46,3 +46,12 @@ def test_refusals_do_not_launch(p1a):
     assert L.p1a_attn_decode(4096, ctypes.byref(kv), 4096, None, 33, 0, None, None, 0, 24, 0.0625, None) == -1  # too many rows
     assert L.p1a_attn_decode(4100, ctypes.byref(kv), 4096, None, 1, 0, None, None, 0, 24, 0.0625, None) == -1   # misaligned q
     assert b"aligned" in L.p1a_last_error()
+
+
+def test_cpp_mirror_header_compiles():
+    """include/p100e_fast_attn.hpp is self-contained C++17 over the C ABI (host compile only, no GPU needed)"""
+    import subprocess
+    src = '#include "p100e_fast_attn.hpp"\nint main() { p100e::fast::kv_cache c; return (int) p100e::fast::kv_row_bytes(c.type, 4, 256) == 2048 ? 0 : 1; }\n'
+    r = subprocess.run(["/opt/rocm/bin/hipcc", "-std=c++17", "-fsyntax-only", "-x", "c++", "-I" + os.path.join(ROOT, "include"),
+                        "-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__", "-"], input=src, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-2000:]
