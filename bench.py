@@ -179,6 +179,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 256 MiB elementwise copy kernel (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU only (no collectives are part of it); run with --gpus 1", file=sys.stderr)
@@ -240,6 +242,13 @@ def main():
                   "kernel_same_pool_GBs": round(step_bytes / sec_kernel_same / 1e9, 1),
                   "merge_kernel_us": round((sec - sec_kernel) * 1e6, 2), "nsplit": p1a.get_nsplit(Hkv)},
     }
+    if args.calib_copy:
+        src = torch.ones(64 * 1024 * 1024, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)                                   # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_extra:
         res["extra"].update(extras(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     if not args.no_cpu:
