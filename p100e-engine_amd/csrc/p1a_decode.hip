@@ -37,12 +37,14 @@ template <uint32_t KT, int D> struct tile_cfg {
     static constexpr int CPK = HB / 16;                        // 16-byte chunks per (key, head)
     static constexpr int NCH = 16 * CPK;                       // chunks per 16-key tile
     static constexpr int NRND = (NCH + 63) / 64;               // load rounds per tile
-    static constexpr int SLOT_B = 16 * HB;                     // one LDS slot: the linear image of 16 head rows
+    static constexpr int TILE_B = 16 * HB;                     // the linear image of 16 head rows
+    static constexpr int QTR_B = 16 * (D / 4) * 4;             // one dim quarter of a wave's accumulators (merge epilogue)
+    static constexpr int SLOT_B = TILE_B > QTR_B ? TILE_B : QTR_B;   // one LDS slot
+    static constexpr int VA_B = KT == P1A_KV_Q4_0 ? 16 * 144 : 0;    // q4_0: 8-byte aligned copy of a V tile's nibbles
     static constexpr int TAB_B = 256;                          // per wave: transposed V scales, later (m, l) of the merge
     static constexpr int NMF = D / 32;                         // QK MFMAs per tile
     static constexpr int NDT = D / 16;                         // output dim tiles
     static_assert(HB % 16 == 0, "head row must be a whole number of 16-byte chunks");
-    static_assert(SLOT_B >= 16 * (D / 4) * 4, "a slot must hold one dim quarter of a wave's accumulators");
 };
 
 #ifdef P1A_TRACE
@@ -86,6 +88,15 @@ __device__ __forceinline__ u2 deq4(uint32_t w, h2 d01, h2 d23) {
     return u2{__builtin_bit_cast(uint32_t, (a - off) * d01), __builtin_bit_cast(uint32_t, (b - off) * d23)};
 }
 
+// 4 nibbles (the low nibbles of the 4 bytes of w) -> ((n - 8) * d) as two packed f16 pairs (0x6400 | n = 1024 + n)
+__device__ __forceinline__ u2 deq4n2(uint32_t w, h2 d01, h2 d23) {
+    const h2 off = {(half_t) 1032, (half_t) 1032};
+    const h2 a = __builtin_bit_cast(h2, perm(0x64646464u, w, 0x04010400u));
+    const h2 b = __builtin_bit_cast(h2, perm(0x64646464u, w, 0x04030402u));
+    return u2{__builtin_bit_cast(uint32_t, (a - off) * d01), __builtin_bit_cast(uint32_t, (b - off) * d23)};
+}
+__device__ __forceinline__ u2 deq4n(uint32_t w, h2 dd) { return deq4n2(w, dd, dd); }
+
 // ---- hand-issued memory operations of the tile ring ----
 // The tile loads are global_load_lds_dwordx4 (global -> LDS, 16 bytes per lane, lane i lands at M0 + 16 i). They are
 // written as inline assembly so that the waits on them can be partial: the vector-memory counter retires in order,
@@ -123,6 +134,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     __shared__ __attribute__((aligned(16))) char vb0[NWV * C::SLOT_B];
     __shared__ __attribute__((aligned(16))) char vb1[NWV * C::SLOT_B];
     __shared__ __attribute__((aligned(16))) char tabs[NWV * C::TAB_B];
+    __shared__ __attribute__((aligned(16))) char vab[NWV * C::VA_B + 16];
 
     const int lane = threadIdx.x & 63, wave = rfl(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
@@ -151,6 +163,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     char * const ks0 = kb0 + wave * C::SLOT_B, * const ks1 = kb1 + wave * C::SLOT_B;
     char * const vs0 = vb0 + wave * C::SLOT_B, * const vs1 = vb1 + wave * C::SLOT_B;
     char * const tab = tabs + wave * C::TAB_B;
+    char * const va = vab + wave * C::VA_B;
 
     // visible-position limit of each of this lane's columns, and the group's maximum
     int plim[NT];
@@ -230,10 +243,13 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         const float * qr = P.q + ((size_t) (row0 + t) * P.Hq + (size_t) hk * P.GQA + hh) * D;
 #pragma unroll
         for (int m = 0; m < C::NMF; ++m) {
-            const int d0 = KT == P1A_KV_F16 ? 32 * m + 8 * g : 16 * (4 * (m >> 1) + g) + 8 * (m & 1);
+            // the 8 dims of k-slot group g of product m: f16 a run of 8; q8_0 half of a 16-code chunk; q4_0 the values
+            // of nibble bytes 4 g .. 4 g + 3 of block m (low nibbles = values 4 g .., high nibbles = values 16 + 4 g ..)
+            const int d0 = KT == P1A_KV_F16 ? 32 * m + 8 * g : KT == P1A_KV_Q8_0 ? 16 * (4 * (m >> 1) + g) + 8 * (m & 1) : 32 * m + 4 * g;
+            const int d1 = KT == P1A_KV_Q4_0 ? d0 + 16 : d0 + 4;
             float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
 #ifndef P1A_EXP_NOQ
-            if (livec) { a = *reinterpret_cast<const float4 *>(qr + d0); b = *reinterpret_cast<const float4 *>(qr + d0 + 4); }
+            if (livec) { a = *reinterpret_cast<const float4 *>(qr + d0); b = *reinterpret_cast<const float4 *>(qr + d1); }
 #else
             a.x = (float) (size_t) qr;
 #endif
@@ -283,6 +299,19 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
                 for (int r = 0; r < NT; ++r) s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[r][m], s[r], 0, 0, 0);
                 if (have_n && m < C::NRND) fetch_round(ksn, kn, tn, m);
             }
+        } else if constexpr (KT == P1A_KV_Q4_0) {   // 8 blocks of 18 B: f16 scale, then 16 nibble bytes (2-byte aligned)
+#pragma unroll
+            for (int b = 0; b < C::NMF; ++b) {
+                const uint16_t * blk = reinterpret_cast<const uint16_t *>(krow + 18 * b);
+                const uint32_t d16 = blk[0];
+                const uint32_t w = (uint32_t) blk[1 + 2 * g] | ((uint32_t) blk[2 + 2 * g] << 16);   // nibble bytes 4 g .. 4 g + 3
+                const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
+                const u2 lo = deq4n(w & 0x0f0f0f0fu, dd), hi = deq4n((w >> 4) & 0x0f0f0f0fu, dd);
+                const u4 a = {lo.lo, lo.hi, hi.lo, hi.hi};
+#pragma unroll
+                for (int r = 0; r < NT; ++r) s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), qf[r][b], s[r], 0, 0, 0);
+                if (have_n && b < C::NRND) fetch_round(ksn, kn, tn, b);
+            }
         } else {   // q8_0: 16 B of scales, then 16 chunks of 16 codes
             const i4 sc = *reinterpret_cast<const i4 *>(krow);
 #pragma unroll
@@ -304,7 +333,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         }
         if (have_n) {   // the rounds the product loop had no place for
 #pragma unroll
-            for (int rd = (KT == P1A_KV_F16 ? C::NMF : C::NMF / 2); rd < C::NRND; ++rd) fetch_round(ksn, kn, tn, rd);
+            for (int rd = (KT == P1A_KV_Q8_0 ? C::NMF / 2 : C::NMF); rd < C::NRND; ++rd) fetch_round(ksn, kn, tn, rd);
         }
 
         // ---- online softmax (log2 domain); column = query row, this lane holds keys ts + 4 g + i ----
@@ -360,6 +389,44 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
                 for (int r = 0; r < NT; ++r) o[r][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[r], o[r][j], 0, 0, 0);
                 if (have_n && j < C::NRND) fetch_round(vsn, vn, tn, j);
             }
+        } else if constexpr (KT == P1A_KV_Q4_0) {
+            {   // re-align: nibble bytes of block bb of a key -> va[key][bb][16] (8-byte aligned for the transposing read);
+                // scales -> tab[block][key]
+                const int key = lane & 15, q2 = lane >> 4;
+#pragma unroll
+                for (int x = 0; x < 2; ++x) {
+                    const int bb = 2 * q2 + x;
+                    const uint16_t * blk = reinterpret_cast<const uint16_t *>(vs + key * C::HB + 18 * bb);
+                    *reinterpret_cast<uint16_t *>(tab + bb * 32 + key * 2) = blk[0];
+                    u4 n;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) n[k] = (uint32_t) blk[1 + 2 * k] | ((uint32_t) blk[2 + 2 * k] << 16);
+                    *reinterpret_cast<u4 *>(va + key * 144 + 16 * bb) = n;
+                }
+            }
+            // one transposing read returns 8 rows: rows 0-3 = keys 4 g .. 4 g + 3, nibble bytes of block 2 p; rows 4-7 =
+            // the same keys, block 2 p + 1. Low nibbles are dims 32 b + c, high nibbles dims 32 b + 16 + c.
+            const int kk = c >> 1, jb = c & 1;
+            const char * vrow = va + (4 * g + (kk & 3)) * 144 + 16 * (kk >> 2) + 8 * jb;
+#pragma unroll
+            for (int p = 0; p < C::NMF / 2; ++p) {
+                const i2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) (vrow + p * 32));
+#pragma unroll
+                for (int x = 0; x < 2; ++x) {
+                    const int b = 2 * p + x;
+                    const h4 dv = *reinterpret_cast<const h4 *>(tab + b * 32 + g * 8);
+                    const uint32_t wx = (uint32_t) w[x];
+                    const u2 lo = deq4n2(wx & 0x0f0f0f0fu, h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
+                    const u2 hi = deq4n2((wx >> 4) & 0x0f0f0f0fu, h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
+                    const i2 a0 = {(int) lo.lo, (int) lo.hi}, a1 = {(int) hi.lo, (int) hi.hi};
+#pragma unroll
+                    for (int r = 0; r < NT; ++r) {
+                        o[r][2 * b] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a0), pb[r], o[r][2 * b], 0, 0, 0);
+                        o[r][2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a1), pb[r], o[r][2 * b + 1], 0, 0, 0);
+                    }
+                }
+                if (have_n && p < C::NRND) fetch_round(vsn, vn, tn, p);
+            }
         } else {
             {   // transposed scale table tab[block][key] (f16, 32 B per block)
                 const int key = lane & 15, q2 = lane >> 4;    // this lane moves blocks 2 q2 and 2 q2 + 1 of its key
@@ -386,7 +453,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
                 if (have_n && j / 2 < C::NRND) fetch_round(vsn, vn, tn, j / 2);
             }
         }
-        static_assert(C::NRND <= (KT == P1A_KV_F16 ? C::NDT : C::NDT / 2), "the PV loop must have room for every V load");
+        static_assert(C::NRND <= (KT == P1A_KV_F16 ? C::NDT : KT == P1A_KV_Q8_0 ? C::NDT / 2 : C::NMF / 2), "the PV loop must have room for every V load");
 #pragma unroll
         for (int r = 0; r < NT; ++r) ol[r] = __builtin_amdgcn_mfma_f32_16x16x16f16(ones, pb[r], ol[r], 0, 0, 0);
     };
@@ -641,8 +708,7 @@ struct dec_plan {
 bool mfma_ok(const p1a_kv & c, int GQA) {
     if (GQA < 1 || GQA > 16) return false;
     if (c.type == P1A_KV_F16) { if (c.D != 64 && c.D != 128 && c.D != 256) return false; }
-    else if (c.type == P1A_KV_Q8_0) { if (c.D != 256) return false; }
-    else return false;
+    else { if (c.D != 256) return false; }   // q8_0 / q4_0 head rows are whole 16-byte chunks only at D = 256
     if (((uintptr_t) c.k | (uintptr_t) c.v) & 15) return false;
     if (c.pt && ((c.pstride & 15) || c.psh < 4)) return false;
     return true;
@@ -736,6 +802,7 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
     int rc;
     if (pl.mfma) {
         if (c.type == P1A_KV_Q8_0) rc = launch_mfma<P1A_KV_Q8_0, 256>(c, a, pl, s);
+        else if (c.type == P1A_KV_Q4_0) rc = launch_mfma<P1A_KV_Q4_0, 256>(c, a, pl, s);
         else if (c.D == 256) rc = launch_mfma<P1A_KV_F16, 256>(c, a, pl, s);
         else if (c.D == 128) rc = launch_mfma<P1A_KV_F16, 128>(c, a, pl, s);
         else rc = launch_mfma<P1A_KV_F16, 64>(c, a, pl, s);
