@@ -33,6 +33,13 @@ template <int D> struct pf_cfg {
     static constexpr int NDT = D / 32;         // 32-dim tiles of O^T
 };
 
+#ifdef P1A_TRACE
+__device__ long long * g_pf_trace = nullptr;   // development build only: per-workgroup phase cycle totals
+#define PT(i) do { const long long t_ = clock64(); acc_t[i] += t_ - last_t; last_t = t_; } while (0)
+#else
+#define PT(i) do { } while (0)
+#endif
+
 struct pf_params {
     const float * q;
     float * out;
@@ -63,6 +70,36 @@ __device__ __forceinline__ pair32 deq4x4(uint32_t w, h2 dd) {
     const h2 b = __builtin_bit_cast(h2, perm_b(0x64646464u, w, 0x04030402u));
     return pair32{__builtin_bit_cast(uint32_t, (a - off) * dd), __builtin_bit_cast(uint32_t, (b - off) * dd)};
 }
+
+// The output accumulators (O^T and the softmax denominator) live in accumulation registers (AGPRs): MFMA reads and
+// writes them there, which leaves the 256 architectural VGPRs to S and the staging data. VALU cannot touch an AGPR, so
+// the (rare) rescale of a column goes through a scratch VGPR by hand. Each accumulator tile is pinned to a fixed AGPR
+// range while it is rescaled (tile n in a[16n : 16n+15]), which lets the assembly name the registers one by one and
+// keeps the register allocator from shuttling all of them through VGPRs on every loop iteration.
+#define P1A_RS1(n) "v_accvgpr_read_b32 %1, a" #n "\n\tv_mul_f32 %1, %1, %2\n\tv_accvgpr_write_b32 a" #n ", %1\n\t"
+#define P1A_RS16(a, b, c, d, e, f, g, h, i, j, k, l, m, n, o, p) \
+    P1A_RS1(a) P1A_RS1(b) P1A_RS1(c) P1A_RS1(d) P1A_RS1(e) P1A_RS1(f) P1A_RS1(g) P1A_RS1(h) \
+    P1A_RS1(i) P1A_RS1(j) P1A_RS1(k) P1A_RS1(l) P1A_RS1(m) P1A_RS1(n) P1A_RS1(o) P1A_RS1(p)
+#define P1A_ACC_SCALE(vec, range, ...)                                                                        \
+    do {                                                                                                      \
+        float t_;                                                                                             \
+        asm volatile(P1A_RS16(__VA_ARGS__) "s_nop 4" : "+{" range "}"(vec), "=&v"(t_) : "v"(alpha));       \
+    } while (0)
+// O^T += A B on a pinned accumulator tile. Consecutive calls name different tiles, so no two dependent MFMAs are ever
+// closer than eight independent ones; the operands come from LDS reads and conversions the compiler has waited for.
+#define P1A_ACC_MFMA(vec, range, a_, b_) \
+    asm volatile("v_mfma_f32_32x32x16_f16 " range ", %1, %2, " range : "+{" range "}"(vec) : "v"(a_), "v"(b_))
+__device__ __forceinline__ float acc_get(float x) {
+#ifndef P1A_PF_PIN
+    return x;
+#endif
+    float t;
+    asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(t) : "a"(x));
+    return t;
+}
+// MFMA results must have left the matrix pipeline before v_accvgpr_read may name them
+__device__ __forceinline__ void acc_settle() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+constexpr float RESCALE_STEP = 8.0f;   // log2 units: the reference maximum of a row only moves in steps larger than this
 
 // ---- per-type staging: raw tile of one kv head -> registers -> f16 rows in LDS ----
 // Every thread owns a fixed set of (key, 16-dim chunk) pairs of the tile; `raw` keeps what was loaded for them.
@@ -216,39 +253,95 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     }
     const h8 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
 
-    // byte offsets of the rows this thread stages, for a tile starting at k0 (keys past pmax are clamped onto pmax)
-    auto rowoffs = [&](int k0, size_t * ro) {
+#ifdef P1A_TRACE
+    long long acc_t[12] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    long long last_t = clock64();
+#endif
+    // Row offsets of a tile. A tile is four groups of 16 keys; with pages of >= 16 positions (or a contiguous cache) a
+    // group lies in one page, so its base is wave-uniform: the page-table entries are fetched once per tile, one tile
+    // ahead of their use, instead of once per thread and key in front of every load. Keys past pmax are clamped onto it.
+    const bool grouped = !ptab || P.pg.psh >= 4;
+    // The table entries are fetched with hand-issued scalar loads (s_load_dword): they do not share the in-order
+    // vector-memory counter with the tile loads in flight, and they are issued where written - one iteration before
+    // rowoffs() waits for them - instead of wherever the scheduler would sink an ordinary load to.
+    const int pmask = (1 << P.pg.psh) - 1;
+    struct gpages { int pg[BN / 16]; };
+    auto group_pages = [&](int k0) {
+        gpages r;
+#pragma unroll
+        for (int gq = 0; gq < BN / 16; ++gq) r.pg[gq] = 0;
+        if (ptab && grouped) {
+#pragma unroll
+            for (int gq = 0; gq < BN / 16; ++gq) {
+                const int32_t * e = ptab + (__builtin_amdgcn_readfirstlane(min(k0 + 16 * gq, pmax)) >> P.pg.psh);
+                asm volatile("s_load_dword %0, %1, 0x0" : "=s"(r.pg[gq]) : "s"(e));
+            }
+        }
+        return r;
+    };
+    auto rowoffs = [&](int k0, gpages & gp, size_t * ro) {
+        size_t go[BN / 16];
+        static_assert(BN / 16 == 4, "the wait below names four entries");
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(gp.pg[0]), "+s"(gp.pg[1]), "+s"(gp.pg[2]), "+s"(gp.pg[3]));
+        PT(9);
+        if (grouped) {
+#pragma unroll
+            for (int gq = 0; gq < BN / 16; ++gq) {
+                const int p = __builtin_amdgcn_readfirstlane(min(k0 + 16 * gq, pmax));
+                go[gq] = (ptab ? (size_t) gp.pg[gq] * P.pg.pstride + (size_t) (p & pmask) * P.pg.rowb : (size_t) p * P.pg.rowb) + head_off;
+            }
+        }
+        PT(10);
 #pragma unroll
         for (int x = 0; x < S::NPT; ++x) {
-            const int i = x * NTHR + tid, key = i / S::CPK;
-            const int p = min(k0 + min(key, BN - 1), pmax);
-            ro[x] = kv_off_tab(P.pg, ptab, p) + head_off;
+            const int i = x * NTHR + tid, key = min(i / S::CPK, BN - 1);
+            if (grouped) {
+                const int gq = key >> 4, room = pmax - (k0 + 16 * gq);      // keys of the group before pmax (< 0: none)
+                size_t base = go[0];
+#pragma unroll
+                for (int j = 1; j < BN / 16; ++j) base = gq == j ? go[j] : base;
+                ro[x] = base + (size_t) (min(key & 15, max(room, 0)) * (int) P.pg.rowb);
+            } else {
+                ro[x] = kv_off_tab(P.pg, ptab, min(k0 + key, pmax)) + head_off;
+            }
         }
     };
 
+    // Workgroups that share a kv head would otherwise walk the keys in lock-step and ask one L2 channel for the same
+    // line at the same instant. Each starts at its own tile and wraps around (softmax does not care about key order);
+    // the q heads of one group stay one tile apart, so all but the first still find the tile in L2.
+    const int rot = (int) (((unsigned) unit * 29u + (unsigned) hh) % (unsigned) ntiles);
+    auto tile_of = [&](int it) { const int t = it + rot; return t >= ntiles ? t - ntiles : t; };
     typename S::raw rk, rv;
     {
         size_t ro[S::NPT];
-        rowoffs(0, ro);
+        gpages g0 = group_pages(tile_of(0) * BN);
+        rowoffs(tile_of(0) * BN, g0, ro);
         S::load(rk, P.kc, ro, tid);
         S::load(rv, P.vc, ro, tid);
     }
+    gpages go_next = group_pages(tile_of(ntiles > 1 ? 1 : 0) * BN);   // pages of the second tile, consumed in iteration 0
     S::store(rk, lds, C::KSTR, tid);
     S::store(rv, lds + C::KT_B, C::VSTR, tid);
     __syncthreads();
 
-    for (int tile = 0; tile < ntiles; ++tile) {
-        const int k0 = tile * BN;
-        char * kt = lds + (tile & 1) * C::STAGE_B;
+    for (int it = 0; it < ntiles; ++it) {
+        const int k0 = tile_of(it) * BN;
+        char * kt = lds + (it & 1) * C::STAGE_B;
         char * vt = kt + C::KT_B;
-        char * nkt = lds + ((tile + 1) & 1) * C::STAGE_B;
-        const bool more = tile + 1 < ntiles;
+        char * nkt = lds + ((it + 1) & 1) * C::STAGE_B;
+        const bool more = it + 1 < ntiles;
+        PT(8);
         if (more) {   // raw loads of the next tile fly while this one is multiplied
             size_t ro[S::NPT];
-            rowoffs(k0 + BN, ro);
+            rowoffs(tile_of(it + 1) * BN, go_next, ro);
+            PT(6);
             S::load(rk, P.kc, ro, tid);
+            PT(7);
             S::load(rv, P.vc, ro, tid);
+            if (it + 2 < ntiles) go_next = group_pages(tile_of(it + 2) * BN);   // page entries needed one iteration on
         }
+        PT(0);
         const bool active = wave_live && k0 <= wave_pmax;     // tiles above this wave's diagonal contribute nothing
         h8 pb[BN / 16];
         if (active) {
@@ -265,6 +358,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                     s[u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qf[ks], s[u], 0, 0, 0);
                 }
             }
+            PT(1);
             // ---- online softmax: this lane holds keys k0 + 32 u + 8 (i / 4) + 4 g + (i % 4) of its own row ----
             float mloc = NEG_INF;
             if (k0 + BN - 1 > wave_pmin) {                     // the tile straddles the diagonal of some row: mask
@@ -281,9 +375,14 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 #pragma unroll
                 for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, s[u][i]);
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-            const float mnew = fmaxf(m_run, mloc);             // finite: key k0 <= wave_pmin... is visible to every live row
+            // Lazy reference maximum: m_run follows the row maximum only when it has grown by more than RESCALE_STEP, so
+            // P stays below 2^RESCALE_STEP (exact in f16 range) and the accumulators are rescaled a handful of times per
+            // row instead of at every tile. A row that has seen no visible key yet (m_run = -inf) just adopts the maximum.
+            const bool fresh = m_run == NEG_INF;
+            const bool move = mloc > m_run + RESCALE_STEP || fresh;      // mloc = -inf never moves anything
+            const float mnew = (move && mloc != NEG_INF) ? mloc : m_run;
             const bool dead = mnew == NEG_INF;
-            const float alpha = (dead || m_run == NEG_INF) ? 1.0f : __builtin_amdgcn_exp2f(m_run - mnew);
+            const float alpha = (fresh || mnew == m_run) ? 1.0f : __builtin_amdgcn_exp2f(m_run - mnew);
             m_run = mnew;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -295,19 +394,38 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                 pb[ps] = h8{(half_t) s[u][b], (half_t) s[u][b + 1], (half_t) s[u][b + 2], (half_t) s[u][b + 3],
                             (half_t) s[u][b + 4], (half_t) s[u][b + 5], (half_t) s[u][b + 6], (half_t) s[u][b + 7]};
             }
-            if (__any(alpha != 1.0f)) {
+            if (__builtin_expect(__any(alpha != 1.0f), 0)) {
+#ifndef P1A_PF_PIN
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     ol[i] *= alpha;
 #pragma unroll
                     for (int dt = 0; dt < C::NDT; ++dt) o[dt][i] *= alpha;
                 }
+#else
+                acc_settle();
+                P1A_ACC_SCALE(o[0], "a[0:15]", 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+                P1A_ACC_SCALE(o[1], "a[16:31]", 16, 17, 18, 19, 20, 21, 22, 23, 24, 25, 26, 27, 28, 29, 30, 31);
+                if constexpr (C::NDT > 2) {
+                    P1A_ACC_SCALE(o[2], "a[32:47]", 32, 33, 34, 35, 36, 37, 38, 39, 40, 41, 42, 43, 44, 45, 46, 47);
+                    P1A_ACC_SCALE(o[3], "a[48:63]", 48, 49, 50, 51, 52, 53, 54, 55, 56, 57, 58, 59, 60, 61, 62, 63);
+                }
+                if constexpr (C::NDT > 4) {
+                    P1A_ACC_SCALE(o[4], "a[64:79]", 64, 65, 66, 67, 68, 69, 70, 71, 72, 73, 74, 75, 76, 77, 78, 79);
+                    P1A_ACC_SCALE(o[5], "a[80:95]", 80, 81, 82, 83, 84, 85, 86, 87, 88, 89, 90, 91, 92, 93, 94, 95);
+                    P1A_ACC_SCALE(o[6], "a[96:111]", 96, 97, 98, 99, 100, 101, 102, 103, 104, 105, 106, 107, 108, 109, 110, 111);
+                    P1A_ACC_SCALE(o[7], "a[112:127]", 112, 113, 114, 115, 116, 117, 118, 119, 120, 121, 122, 123, 124, 125, 126, 127);
+                }
+                P1A_ACC_SCALE(ol, "a[128:143]", 128, 129, 130, 131, 132, 133, 134, 135, 136, 137, 138, 139, 140, 141, 142, 143);
+#endif
             }
         }
+        PT(2);
         if (more) {   // convert the next tile into the other buffer
             S::store(rk, nkt, C::KSTR, tid);
             S::store(rv, nkt + C::KT_B, C::VSTR, tid);
         }
+        PT(3);
         if (active) {
             // ---- O^T += V^T P^T. Slot e of lane half g in k-step ps is key 16 ps + 4 g + e (e < 4) or 16 ps + 8 + 4 g + e - 4 ----
             const int i16 = lane & 15, blk = lane >> 4;        // 16-lane block: dims 16 (blk & 1) .., lane half blk >> 1 == g
@@ -322,17 +440,42 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                     const s4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + 8 * C::VSTR));
                     const h4 l4 = __builtin_bit_cast(h4, lo), h4_ = __builtin_bit_cast(h4, hi);
                     const h8 a = {l4[0], l4[1], l4[2], l4[3], h4_[0], h4_[1], h4_[2], h4_[3]};
+#ifndef P1A_PF_PIN
                     o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[ps], o[dt], 0, 0, 0);
                 }
                 ol = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[ps], ol, 0, 0, 0);
             }
+#else
+                    if (dt == 0) P1A_ACC_MFMA(o[0], "a[0:15]", a, pb[ps]);
+                    if (dt == 1) P1A_ACC_MFMA(o[1], "a[16:31]", a, pb[ps]);
+                    if constexpr (C::NDT > 2) {
+                        if (dt == 2) P1A_ACC_MFMA(o[2], "a[32:47]", a, pb[ps]);
+                        if (dt == 3) P1A_ACC_MFMA(o[3], "a[48:63]", a, pb[ps]);
+                    }
+                    if constexpr (C::NDT > 4) {
+                        if (dt == 4) P1A_ACC_MFMA(o[4], "a[64:79]", a, pb[ps]);
+                        if (dt == 5) P1A_ACC_MFMA(o[5], "a[80:95]", a, pb[ps]);
+                        if (dt == 6) P1A_ACC_MFMA(o[6], "a[96:111]", a, pb[ps]);
+                        if (dt == 7) P1A_ACC_MFMA(o[7], "a[112:127]", a, pb[ps]);
+                    }
+                }
+                P1A_ACC_MFMA(ol, "a[128:143]", ones, pb[ps]);
+            }
+#endif
+            acc_settle();   // the compiler does not know these are MFMAs: let them retire before it may copy a tile
         }
+        PT(4);
         __syncthreads();
+        PT(5);
     }
+#ifdef P1A_TRACE
+    if (g_pf_trace && tid == 0) for (int i = 0; i < 12; ++i) g_pf_trace[(size_t) blockIdx.x * 12 + i] = acc_t[i];
+#endif
 
     // ---- epilogue: normalise, gate, store. Lane (row c, half g) holds dims 32 dt + 8 (i / 4) + 4 g + (i % 4) ----
     if (live) {
-        const float inv = 1.0f / ol[0];
+        acc_settle();
+        const float inv = 1.0f / acc_get(ol[0]);
         float * orow = P.out + ((size_t) my_tok * P.Hq + h) * D;
         const float * grow = P.gate ? P.gate + ((size_t) my_tok * P.Hq + h) * D : nullptr;
 #pragma unroll
@@ -340,7 +483,8 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
                 const int d0 = 32 * dt + 8 * q4 + 4 * g;
-                f4 r = {o[dt][4 * q4] * inv, o[dt][4 * q4 + 1] * inv, o[dt][4 * q4 + 2] * inv, o[dt][4 * q4 + 3] * inv};
+                f4 r = {acc_get(o[dt][4 * q4]) * inv, acc_get(o[dt][4 * q4 + 1]) * inv, acc_get(o[dt][4 * q4 + 2]) * inv,
+                        acc_get(o[dt][4 * q4 + 3]) * inv};
                 if (grow) {
                     const f4 gt = *reinterpret_cast<const f4 *>(grow + d0);
 #pragma unroll
@@ -390,6 +534,10 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
 }
 
 }   // namespace p1a
+
+#ifdef P1A_TRACE
+extern "C" void p1a_set_pf_trace(long long * buf) { (void) hipMemcpyToSymbol(HIP_SYMBOL(p1a::g_pf_trace), &buf, sizeof buf); }
+#endif
 
 extern "C" size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D) {
     (void) T; (void) p0; (void) Hq; (void) Hkv; (void) D;
