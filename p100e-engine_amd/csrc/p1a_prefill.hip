@@ -82,27 +82,40 @@ constexpr float RESCALE_STEP = 8.0f;   // log2 units: the reference maximum of a
 // gb[x] + vo[x][n]: gb = cache base + the base of the item's 16-key group (wave-uniform whenever 16 * CPK is a multiple
 // of the wave size, so it sits in scalar registers), vo = the loop-invariant 32-bit offset of the item inside its group
 // (row in the group * row bytes + offs()[n]); the loads then need no address arithmetic at all.
+typedef unsigned u2v __attribute__((ext_vector_type(2)));
+typedef uint32_t __attribute__((may_alias)) u32a;   // the parked scale blocks are written as dwords and read as halves
+typedef uint16_t __attribute__((may_alias)) u16a;
 typedef const __attribute__((address_space(1))) char * gptr;      // global memory, so the loads are global_load (vmcnt only)
 #define P1A_GLOAD(T, p) (*(const __attribute__((address_space(1))) T *) (p))
 template <uint32_t KT, int D> struct stager;
+// Which (key, chunk) of the 64-key tile item x of thread tid is. Wave-major whenever the chunks of a key divide a wave
+// evenly: wave w owns keys 16 w .. 16 w + 15 - exactly one 16-key group, so one page base serves all its loads - and
+// item x covers KPW = 64 / CPK of them. (Otherwise: items dealt out thread by thread over the whole tile.)
+template <int CPK> struct item_map {
+    static constexpr bool WAVE_MAJOR = CPK % 4 == 0 && CPK <= 64;
+    static constexpr int KPW = WAVE_MAJOR ? 64 / CPK : 1;
+    static __device__ __forceinline__ int key(int x, int tid) { return WAVE_MAJOR ? 16 * (tid >> 6) + x * KPW + (tid & 63) / CPK : (x * NTHR + tid) / CPK; }
+    static __device__ __forceinline__ int cc(int x, int tid) { return WAVE_MAJOR ? (tid & 63) % CPK : (x * NTHR + tid) % CPK; }
+};
 
 template <int D> struct stager<P1A_KV_Q8_0, D> {
     static constexpr int CPK = D / 16;                    // 16-code chunks per key
     static constexpr int NPT = BN * CPK / NTHR;           // items per thread
-    static constexpr int NOFF = 2;                        // codes, scale
+    static constexpr int NOFF = 1;                        // codes
+    // Sub-dword loads cost twice the issue time of a 16-byte one, so an item does not fetch its own f16 scale: each wave
+    // fetches the scale blocks (D/32 scales) of the 16 keys its items belong to with ONE load per tile, parks them in a
+    // small LDS area of its own and every lane picks its scales up from there.
+    static constexpr bool SCALES_VIA_LDS = true;
+    static constexpr int SB = (D / 32) * 2;               // bytes of scales per key head
     static_assert(BN * CPK % NTHR == 0, "tile must split evenly over the threads");
-    struct raw { u4 w[NPT]; uint16_t d[NPT]; };
-    static __device__ __forceinline__ void offs(uint32_t * o, int cc) { o[0] = (D / 32) * 2 + cc * 16; o[1] = (cc >> 1) * 2; }
-    static __device__ __forceinline__ void load(raw & r, const gptr * gb, const uint32_t (*vo)[NOFF], int) {
-#pragma unroll
-        for (int x = 0; x < NPT; ++x) {
-            r.w[x] = P1A_GLOAD(u4, gb[x] + vo[x][0]);
-            r.d[x] = P1A_GLOAD(uint16_t, gb[x] + vo[x][1]);
-        }
+    struct raw { u4 w[NPT]; uint32_t d[NPT]; };           // d: one zero-extended f16 scale per item
+    static __device__ __forceinline__ void offs(uint32_t * o, int cc) { o[0] = (D / 32) * 2 + cc * 16; }
+    static __device__ __forceinline__ void load_item(raw & r, gptr gb, const uint32_t * vo, int x, int) {
+        r.w[x] = P1A_GLOAD(u4, gb + vo[0]);
     }
     static constexpr int PARTS = 2;                       // 16-byte LDS stores per item
     static __device__ __forceinline__ void store_part(const raw & r, char * tile, int stride, int tid, int x, int part) {
-        const int i = x * NTHR + tid, key = i / CPK, cc = i - key * CPK;
+        const int key = item_map<CPK>::key(x, tid), cc = item_map<CPK>::cc(x, tid);
         const uint32_t d16 = r.d[x];
         const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
         const pair32 x0 = deq8x4(r.w[x][2 * part], dd), x1 = deq8x4(r.w[x][2 * part + 1], dd);
@@ -114,16 +127,17 @@ template <int D> struct stager<P1A_KV_F16, D> {
     static constexpr int CPK = D / 8;                     // 16-byte chunks (8 halves) per key
     static constexpr int NPT = BN * CPK / NTHR;
     static constexpr int NOFF = 1;
+    static constexpr bool SCALES_VIA_LDS = false;
+    static constexpr int SB = 4;
     static_assert(BN * CPK % NTHR == 0, "tile must split evenly over the threads");
     struct raw { u4 w[NPT]; };
     static __device__ __forceinline__ void offs(uint32_t * o, int cc) { o[0] = cc * 16; }
-    static __device__ __forceinline__ void load(raw & r, const gptr * gb, const uint32_t (*vo)[NOFF], int) {
-#pragma unroll
-        for (int x = 0; x < NPT; ++x) r.w[x] = P1A_GLOAD(u4, gb[x] + vo[x][0]);
+    static __device__ __forceinline__ void load_item(raw & r, gptr gb, const uint32_t * vo, int x, int) {
+        r.w[x] = P1A_GLOAD(u4, gb + vo[0]);
     }
     static constexpr int PARTS = 1;
     static __device__ __forceinline__ void store_part(const raw & r, char * tile, int stride, int tid, int x, int) {
-        const int i = x * NTHR + tid, key = i / CPK, cc = i - key * CPK;
+        const int key = item_map<CPK>::key(x, tid), cc = item_map<CPK>::cc(x, tid);
         *reinterpret_cast<u4 *>(tile + key * stride + cc * 16) = r.w[x];
     }
 };
@@ -132,22 +146,21 @@ template <int D> struct stager<P1A_KV_Q4_0, D> {
     static constexpr int CPK = D / 32;                    // 18-byte blocks per key: one block (32 values) per item
     static constexpr int NPT = (BN * CPK + NTHR - 1) / NTHR;
     static constexpr int NOFF = 1;
+    static constexpr bool SCALES_VIA_LDS = false;
+    static constexpr int SB = 4;
     struct raw { uint16_t h[NPT][9]; };
     static __device__ __forceinline__ void offs(uint32_t * o, int cc) { o[0] = cc * 18; }
-    static __device__ __forceinline__ void load(raw & r, const gptr * gb, const uint32_t (*vo)[NOFF], int tid) {
+    static __device__ __forceinline__ void load_item(raw & r, gptr gb, const uint32_t * vo, int x, int tid) {
+        const int key = item_map<CPK>::key(x, tid);
+        if (BN * CPK % NTHR == 0 || key < BN) {
+            const gptr blk = gb + vo[0];   // 2-byte aligned
 #pragma unroll
-        for (int x = 0; x < NPT; ++x) {
-            const int i = x * NTHR + tid, key = i / CPK;
-            if (BN * CPK % NTHR == 0 || key < BN) {
-                const gptr blk = gb[x] + vo[x][0];   // 2-byte aligned
-#pragma unroll
-                for (int k = 0; k < 9; ++k) r.h[x][k] = P1A_GLOAD(uint16_t, blk + 2 * k);
-            }
+            for (int k = 0; k < 9; ++k) r.h[x][k] = P1A_GLOAD(uint16_t, blk + 2 * k);
         }
     }
     static constexpr int PARTS = 4;                       // part 0, 1: values 0..15 (low nibbles), part 2, 3: values 16..31
     static __device__ __forceinline__ void store_part(const raw & r, char * tile, int stride, int tid, int x, int part) {
-        const int i = x * NTHR + tid, key = i / CPK, b = i - key * CPK;
+        const int key = item_map<CPK>::key(x, tid), b = item_map<CPK>::cc(x, tid);
         if (!(BN * CPK % NTHR == 0 || key < BN)) return;
         const uint32_t d16 = r.h[x][0];
         const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
@@ -171,7 +184,8 @@ template <class S> __device__ __forceinline__ void store_tile(const typename S::
         for (int part = 0; part < S::PARTS; ++part) S::store_part(r, tile, stride, tid, x, part);
 }
 
-template <uint32_t KT, int D>
+// GROUPED: pages hold at least 16 positions (or the cache is contiguous), so a 16-key group has one base
+template <uint32_t KT, int D, bool GROUPED>
 __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     using C = pf_cfg<D>;
     using S = stager<KT, D>;
@@ -228,20 +242,20 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     const h8 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
 
     // ---- addressing of the raw tile ----
-    // A tile is four groups of 16 keys. With pages of >= 16 positions (or a contiguous cache) a group lies in one page,
-    // so its base is uniform: four page-table entries per tile, fetched with hand-issued scalar loads (s_load_dword does
-    // not share the in-order vector-memory counter with the tile loads in flight) well before the bases are formed.
-    // Inside its group an item sits at a loop-invariant offset; only the tile that holds pmax clamps the rows past it
-    // (they would otherwise read rows nobody has written), and that tile's offsets are prepared once, up front.
-    const bool grouped = !ptab || P.pg.psh >= 4;
+    // A tile is four groups of 16 keys, one per wave. With pages of >= 16 positions (or a contiguous cache) a group lies
+    // in one page, so its base is a scalar: one page-table entry per wave and tile, fetched with a hand-issued scalar
+    // load (s_load_dword does not share the in-order vector-memory counter with the tile loads in flight) well before the
+    // base is formed. Inside the group an item sits at a loop-invariant offset; only the tile that holds pmax clamps the
+    // rows past it (they would otherwise read rows nobody has written); that tile's offsets are prepared once, up front.
+    constexpr bool grouped = GROUPED;
     const int pmask = (1 << P.pg.psh) - 1;
     const int last_tile = ntiles - 1;
-    constexpr bool UNIFORM_GROUP = (16 * S::CPK) % 64 == 0;      // all lanes of a wave work on one group per item
+    using IM = item_map<S::CPK>;
     uint32_t voff[S::NPT][S::NOFF], voff_last[S::NPT][S::NOFF];
-    int grp[S::NPT];
+    int grp[S::NPT];                                             // (wave-major: all equal to the wave number)
 #pragma unroll
     for (int x = 0; x < S::NPT; ++x) {
-        const int i = x * NTHR + tid, key = min(i / S::CPK, BN - 1), cc = i - (i / S::CPK) * S::CPK;
+        const int key = min(IM::key(x, tid), BN - 1), cc = IM::cc(x, tid);
         grp[x] = key >> 4;
         uint32_t co[S::NOFF];
         S::offs(co, cc);
@@ -253,58 +267,97 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             voff_last[x][n] = (uint32_t) kl * (uint32_t) P.pg.rowb + co[n];
         }
     }
-    struct gpages { int pg[BN / 16]; };
-    struct gbases { size_t go[BN / 16]; };
+    // FAST: the wave's 16 keys of a tile lie in one page (or the cache is contiguous): one table entry, one scalar base
+    constexpr bool FAST = GROUPED && IM::WAVE_MAJOR;
+    struct gpages { int pg; };
+    struct gbases { size_t go; };
     auto group_pages = [&](int tile) {
         gpages r;
-#pragma unroll
-        for (int gq = 0; gq < BN / 16; ++gq) r.pg[gq] = 0;
-        if (ptab && grouped) {
-#pragma unroll
-            for (int gq = 0; gq < BN / 16; ++gq) {
-                const int32_t * e = ptab + (__builtin_amdgcn_readfirstlane(min(tile * BN + 16 * gq, pmax)) >> P.pg.psh);
-                asm volatile("s_load_dword %0, %1, 0x0" : "=s"(r.pg[gq]) : "s"(e));
-            }
+        r.pg = 0;
+        if (FAST && ptab) {
+            const int32_t * e = ptab + (__builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, pmax)) >> P.pg.psh);
+            asm volatile("s_load_dword %0, %1, 0x0" : "=s"(r.pg) : "s"(e));
         }
         return r;
     };
     auto group_bases = [&](int tile, gpages & gp) {
         gbases r;
-        static_assert(BN / 16 == 4, "the wait below names four entries");
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(gp.pg[0]), "+s"(gp.pg[1]), "+s"(gp.pg[2]), "+s"(gp.pg[3]));
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(gp.pg));
+        const int p = __builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, pmax));
+        r.go = (ptab ? (size_t) gp.pg * P.pg.pstride + (size_t) (p & pmask) * P.pg.rowb : (size_t) p * P.pg.rowb) + head_off;
+        return r;
+    };
+    // where item x of `tile` starts: base (scalar registers when GROUPED) + 32-bit offsets
+    struct iaddr { gptr base; uint32_t vo[S::NOFF]; };
+    auto item_addr = [&](const char * cache, int tile, const gbases & gb, int x) {
+        iaddr r;
+        if constexpr (FAST) {
+            r.base = (gptr) cache + gb.go;
+            const bool is_last = tile == last_tile;
 #pragma unroll
-        for (int gq = 0; gq < BN / 16; ++gq) {
-            const int p = __builtin_amdgcn_readfirstlane(min(tile * BN + 16 * gq, pmax));
-            r.go[gq] = (ptab ? (size_t) gp.pg[gq] * P.pg.pstride + (size_t) (p & pmask) * P.pg.rowb : (size_t) p * P.pg.rowb) + head_off;
+            for (int n = 0; n < S::NOFF; ++n) r.vo[n] = is_last ? voff_last[x][n] : voff[x][n];
+        } else {   // pages shorter than a group (or items not dealt out wave by wave): every key looks its page up
+            const int key = min(IM::key(x, tid), BN - 1);
+            r.base = (gptr) cache + (kv_off_tab(P.pg, ptab, min(tile * BN + key, pmax)) + head_off);
+#pragma unroll
+            for (int n = 0; n < S::NOFF; ++n) r.vo[n] = voff[x][n] - (uint32_t) (key & 15) * (uint32_t) P.pg.rowb;
         }
         return r;
     };
     auto load_tile = [&](typename S::raw & r, const char * cache, int tile, const gbases & gb) {
-        gptr base[S::NPT];
-        uint32_t vo[S::NPT][S::NOFF];
-        const gptr gcache = (gptr) cache;
-        if (grouped) {
-            const bool is_last = tile == last_tile;
 #pragma unroll
-            for (int x = 0; x < S::NPT; ++x) {
-                const int gq = UNIFORM_GROUP ? __builtin_amdgcn_readfirstlane(grp[x]) : grp[x];
-                size_t off = gb.go[0];
-#pragma unroll
-                for (int j = 1; j < BN / 16; ++j) off = gq == j ? gb.go[j] : off;
-                base[x] = gcache + off;
-#pragma unroll
-                for (int n = 0; n < S::NOFF; ++n) vo[x][n] = is_last ? voff_last[x][n] : voff[x][n];
-            }
-        } else {   // pages shorter than a group: every key looks its page up
-#pragma unroll
-            for (int x = 0; x < S::NPT; ++x) {
-                const int i = x * NTHR + tid, key = min(i / S::CPK, BN - 1);
-                base[x] = gcache + (kv_off_tab(P.pg, ptab, min(tile * BN + key, pmax)) + head_off);
-#pragma unroll
-                for (int n = 0; n < S::NOFF; ++n) vo[x][n] = voff[x][n] - (uint32_t) (key & 15) * (uint32_t) P.pg.rowb;
-            }
+        for (int x = 0; x < S::NPT; ++x) {
+            const iaddr ia = item_addr(cache, tile, gb, x);
+            S::load_item(r, ia.base, ia.vo, x, tid);
         }
-        S::load(r, base, vo, tid);
+    };
+
+    // ---- scale blocks (types that keep their scales apart from the codes) ----
+    // Lane l of a wave (l mod 16) fetches the block of the l-th of the wave's 16 keys; all four quarters of the wave fetch
+    // and park the same 16 blocks, which saves masking lanes off.
+    constexpr bool SVL = S::SCALES_VIA_LDS;
+    static_assert(!SVL || IM::WAVE_MAJOR, "parked scale blocks are per wave");
+    constexpr int KPW = IM::KPW;
+    struct sblk { uint32_t w[S::SB / 4]; };
+    const int l16 = lane & 15;
+    const int lkey = 16 * wave + l16;
+    const uint32_t sb_full = (uint32_t) l16 * (uint32_t) P.pg.rowb;
+    const uint32_t sb_last = (uint32_t) min(l16, max(pmax - (last_tile * BN + 16 * wave), 0)) * (uint32_t) P.pg.rowb;
+    char * const ksc = lds + 2 * C::STAGE_B + wave * 16 * S::SB;           // this wave's parking area: K blocks
+    char * const vsc = ksc + 4 * 16 * S::SB;                               // ... V blocks
+    auto load_sblk = [&](const char * cache, int tile, const gbases & gb) {
+        sblk r;
+        size_t off;
+        if constexpr (FAST) {
+            off = gb.go + (tile == last_tile ? sb_last : sb_full);
+        } else {
+            off = kv_off_tab(P.pg, ptab, min(tile * BN + lkey, pmax)) + head_off;
+        }
+        const gptr p_ = (gptr) cache + off;
+        if constexpr (S::SB == 16) { const u4 t = P1A_GLOAD(u4, p_); r.w[0] = t[0]; r.w[1] = t[1]; r.w[2] = t[2]; r.w[3] = t[3]; }
+        else if constexpr (S::SB == 8) { const u2v t = P1A_GLOAD(u2v, p_); r.w[0] = t[0]; r.w[1] = t[1]; }
+        else r.w[0] = P1A_GLOAD(uint32_t, p_);
+        return r;
+    };
+    auto park_sblk = [&](char * area, const sblk & b) {
+#pragma unroll
+        for (int j = 0; j < S::SB / 4; ++j) reinterpret_cast<u32a *>(area + l16 * S::SB)[j] = b.w[j];
+    };
+    auto pick_scales = [&](typename S::raw & r, const char * area) {
+        if constexpr (SVL) {
+#pragma unroll
+            for (int x = 0; x < S::NPT; ++x)
+                r.d[x] = *reinterpret_cast<const u16a *>(area + (x * KPW + lane / S::CPK) * S::SB + ((lane % S::CPK) >> 1) * 2);
+        }
+    };
+    // prologue helper: a whole raw tile, scales included
+    auto fetch_tile = [&](typename S::raw & r, const char * cache, char * area, int tile, const gbases & gb) {
+        load_tile(r, cache, tile, gb);
+        if constexpr (SVL) {
+            const sblk b = load_sblk(cache, tile, gb);
+            park_sblk(area, b);
+            pick_scales(r, area);
+        }
     };
 
     // Workgroups that share a kv head would otherwise walk the keys in lock-step and ask one L2 channel for the same
@@ -331,19 +384,21 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 
     // ---- prologue: K(0), V(0), K(1) in LDS; V(1) and K(2) on their way in registers; S^T(0) ----
     typename S::raw rk, rv;
+    sblk sk, sv;                                           // scale blocks that belong to rk, rv
     gbases gb_prev;                                        // group bases of the tile whose V is fetched next
     {
         gpages g0 = group_pages(tile_of(0)), g1 = group_pages(tile_of(1)), g2 = group_pages(tile_of(2));
         const gbases b0 = group_bases(tile_of(0), g0), b1 = group_bases(tile_of(1), g1);
         gb_prev = group_bases(tile_of(2), g2);
-        load_tile(rk, P.kc, tile_of(0), b0);
-        load_tile(rv, P.vc, tile_of(0), b0);
+        fetch_tile(rk, P.kc, ksc, tile_of(0), b0);
+        fetch_tile(rv, P.vc, vsc, tile_of(0), b0);
         store_tile<S>(rk, lds, C::KSTR, tid);
         store_tile<S>(rv, lds + C::KT_B, C::VSTR, tid);
-        load_tile(rk, P.kc, tile_of(1), b1);
-        load_tile(rv, P.vc, tile_of(1), b1);
+        fetch_tile(rk, P.kc, ksc, tile_of(1), b1);
         store_tile<S>(rk, lds + C::STAGE_B, C::KSTR, tid);
+        load_tile(rv, P.vc, tile_of(1), b1);
         load_tile(rk, P.kc, tile_of(2), gb_prev);
+        if constexpr (SVL) { sv = load_sblk(P.vc, tile_of(1), b1); sk = load_sblk(P.kc, tile_of(2), gb_prev); }
     }
     __syncthreads();
     f16x s_next[2];
@@ -420,6 +475,10 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 #pragma unroll
         for (int k = HALF; k < NQK; ++k) {
             qk_step(fr, k);
+            if constexpr (SVL) {   // the scales of the raw tiles fetched one step ago: through LDS to the lanes that use them
+                if (k == NQK - 4) { park_sblk(ksc, sk); park_sblk(vsc, sv); }
+                if (k == NQK - 2) { pick_scales(rk, ksc); pick_scales(rv, vsc); }
+            }
 #pragma unroll
             for (int v = 0; v < VPS; ++v) {
                 const int idx = (k - HALF) * VPS + v, su = idx >> 4, i = idx & 15;
@@ -474,16 +533,17 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         }
 
         PT(3);
-        // ---- raw loads of K(it+3), V(it+2): one whole step to arrive ----
+        // ---- raw loads of K(it+3), V(it+2): one whole step to arrive. Issued back to back: a vector memory instruction
+        // holds the wave for as long as the CU's address path needs for it, wherever it is placed ----
         {
             const gbases gb_k = group_bases(tile_of(it + 3), gp_k);
             load_tile(rk, P.kc, tile_of(it + 3), gb_k);
             load_tile(rv, P.vc, tile_of(it + 2), gb_prev);
+            if constexpr (SVL) { sk = load_sblk(P.kc, tile_of(it + 3), gb_k); sv = load_sblk(P.vc, tile_of(it + 2), gb_prev); }
             gb_prev = gb_k;
         }
-        // LDS stores retired, then the barrier. Not __syncthreads(): its fence would also wait for the raw loads just
-        // issued, which have the whole next step to arrive.
         PT(4);
+        // LDS stores retired, then the barrier (without the global-memory fence of __syncthreads())
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         PT(5);
     }
@@ -512,13 +572,13 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     }
 }
 
-template <uint32_t KT, int D>
-int launch_pf(const pf_params & P, hipStream_t s) {
+template <uint32_t KT, int D, bool GROUPED>
+int launch_pf_g(const pf_params & P, hipStream_t s) {
     using C = pf_cfg<D>;
-    const int lds = 2 * C::STAGE_B;
+    const int lds = 2 * C::STAGE_B + (stager<KT, D>::SCALES_VIA_LDS ? 2 * 4 * 16 * stager<KT, D>::SB : 0);
     static bool attr_set = false;
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void *) prefill_k<KT, D>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+        if (hipFuncSetAttribute((const void *) prefill_k<KT, D, GROUPED>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
             (void) hipGetLastError();
             set_error("p1a_attn_prefill: cannot reserve %d bytes of LDS", lds);
             return P1A_E_LAUNCH;
@@ -527,8 +587,12 @@ int launch_pf(const pf_params & P, hipStream_t s) {
     }
     const int units = P.nblk * P.Hkv;
     const int slots = ((units + 7) / 8) * P.GQA;
-    prefill_k<KT, D><<<slots * 8, NTHR, lds, s>>>(P);
+    prefill_k<KT, D, GROUPED><<<slots * 8, NTHR, lds, s>>>(P);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
+}
+template <uint32_t KT, int D>
+int launch_pf(const pf_params & P, hipStream_t s) {
+    return !P.pg.pt || P.pg.psh >= 4 ? launch_pf_g<KT, D, true>(P, s) : launch_pf_g<KT, D, false>(P, s);
 }
 
 }   // namespace
