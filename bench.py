@@ -115,6 +115,16 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
     ab = 2 * T * Hkv * D * 4 + 2 * T * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
     ex["append_T4096_q8_0_us"] = round(sec * 1e6, 2)
     ex["append_GBs"] = round(ab / sec / 1e9, 1)
+    # the input prep of a 4-row verify step (q | gate split, norm, rope, quantizing write) in front of the decode
+    qg4 = torch.randn((4, Hq, 2 * D), generator=g, device="cuda")
+    w_q = torch.ones(D, device="cuda")
+    w_k = torch.ones(D, device="cuda")
+    pos4 = torch.arange(p0, p0 + 4, dtype=torch.int32, device="cuda")
+    q4 = torch.empty((4, Hq, D), device="cuda")
+    g4 = torch.empty((4, Hq * D), device="cuda")
+    with torch.cuda.stream(stream):
+        sec = time_graph(torch, stream, [lambda: p1a.attn_prep(qg4, kc, vc, w_q, w_k, pos4, q4, g4, c, p0, 4, Hq, 64, 1e7, 1e-6)] * 20, 2)
+    ex["prep_4rows_q8_0_us"] = round(sec * 1e6, 2)
     del kv, c, q, gate, out
     # configs[3]: MTP verify, 4 sequences x 4 rows, q4_0, ctx 65536
     n4 = 65536

@@ -2,7 +2,7 @@
 //
 // Same names, argument order, defaults and error behaviour as the reference headers (paths relative to the reference
 // tree): src/fast/attn.cuh:12-70, src/fast/attn_dec2.cuh:17-21, src/fast/attn_fold.cuh:18-26. cudaStream_t becomes
-// hipStream_t; everything is a thin inline call into the C ABI of include/p1a_attn.h (libp1a_attn.so), so a caller
+// hipStream_t; src/fast/fused.cuh:101-113 (attn_prep) is mirrored too; everything is a thin inline call into the C ABI of include/p1a_attn.h (libp1a_attn.so), so a caller
 // that links the reference's static library p100e_fast_attn can link this instead without touching its call sites.
 // Additions, all optional: a trailing `gate` argument (fused sigmoid output gate; nullptr = the reference's
 // behaviour) and `rows_per_seq` on attn_decode_rows (verify blocks that share one KV read).
@@ -78,6 +78,15 @@ inline void kv_append_dev(kv_cache & c, const float * k, const float * v, const 
 inline bool kv_append_rows(kv_cache & c, const float * k, const float * v, const int32_t * pos, int T, hipStream_t s) {
     const p1a_kv p = detail::pod(c);
     return p1a_kv_append(&p, k, v, -1, nullptr, pos, T, s) == P1A_OK;
+}
+
+// src/fast/fused.cuh:101-113 (Hkv and D must be the cache's; the interleaved M-RoPE argument is not mirrored)
+inline bool attn_prep(const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
+                      const int32_t * pos, float * q, float * gate, kv_cache & c, int p0, int T, int Hq, int Hkv, int D,
+                      int n_rot, float freq_base, float eps, hipStream_t s, int ldq = 0, int ldk = 0, int ldv = 0) {
+    if (Hkv != c.Hkv || D != c.D) return false;
+    const p1a_kv p = detail::pod(c);
+    return p1a_attn_prep(qg, k, v, q_norm, k_norm, pos, q, gate, &p, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, s) == P1A_OK;
 }
 
 // src/fast/attn.cuh:39-44. false = nothing launched, out untouched.

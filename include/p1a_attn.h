@@ -78,6 +78,22 @@ int p1a_kv_append(const p1a_kv *c, const float *k, const float *v, int p0, const
                   const int32_t *pos_rows, int T, void *stream);
 
 /*
+ * Attention-layer input prep in one launch: per token t
+ *     qg [T][ldq] (Hq heads, each D floats of q followed by D floats of gate) -> gate [T][Hq*D] (copy) and
+ *                                                                                q [T][Hq][D] = rope(rmsnorm(q) * q_norm)
+ *     k  [T][ldk] (Hkv heads of D) -> rope(rmsnorm(k) * k_norm) -> K cache row;   v [T][ldv] -> V cache row
+ * with rmsnorm(x) = x / sqrt(mean(x^2) + eps) per head, the NEOX rotation of dims (j, j + n_rot/2), j < n_rot/2, by
+ * pos[t] * freq_base^(-2j/n_rot), and the quantizing write of p1a_kv_append. The cache row of token t is p0 + t, or
+ * pos[t] (read on the device, own page table pt + rtab[t]) when p0 < 0; the rotary position is pos[t] in both cases.
+ * ld* = 0 means dense rows; q_norm / k_norm ([D]) may be NULL. D <= 256, n_rot % 8 == 0; interleaved M-RoPE is not covered.
+ * Replaces the front half of attn_prep (src/fast/fused.cuh:101-113, kernel src/fast/fused.cu:512-573) = k::split_q_gate
+ * + fast::rmsnorm + k::rope_neox + kv_append of the unfused path (src/tp_model.cu:1717-1734).
+ */
+int p1a_attn_prep(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
+                  const int32_t *pos, float *q, float *gate, const p1a_kv *c, int p0, int T, int Hq, int n_rot,
+                  float freq_base, float eps, int ldq, int ldk, int ldv, void *stream);
+
+/*
  * Decode / MTP-verify attention: q, out [T][Hq][D] f32;
  *     out[t][h] = softmax_{j <= pos(t)} (scale * q[t][h] . K[j][h / (Hq/Hkv)]) . V[j][h / (Hq/Hkv)]
  * and, when gate != NULL (gate [T][Hq*D] f32), out *= 1 / (1 + exp(-gate)) fused into the final merge.

@@ -184,6 +184,85 @@ void orc_rmsnorm_heads(float *x, size_t nheads, int D, float eps) {
     }
 }
 
+/*
+ * Attention-layer input prep, the front half of the engine's attn_prep (src/fast/fused.cuh:101-113, kernel
+ * src/fast/fused.cu:512-573): per token t and head,
+ *   q heads : gate[t][h] = second half of the head's (q | gate) slice of qg (src/kernels.cu:95-106), then
+ *             q[t][h] = rope(rmsnorm(first half) * q_norm);
+ *   k heads : rope(rmsnorm(k) * k_norm) -> quantized K row of the cache; v heads: raw v -> V row (kv_q8.cuh:20-49);
+ * cache row of token t = pos[t] when p0 < 0, else p0 + t; the ROTARY position is pos[t] in both cases (fused.cu:548).
+ * RMS norm: src/kernels.cu:34-42 / fused.cu:540-550 (x * rsqrt(mean(x^2) + eps) * w); NEOX rope on the first n_rot
+ * dims: pairs (j, j + n_rot/2), theta = pos * freq_base^(-2j/n_rot) (fused.cu:553-562).
+ * The order of the floating-point operations is FIXED here (and the GPU kernel keeps the same order, so that the K
+ * codes can be compared bit for bit): the sum of squares is formed per group of 4 consecutive dims, left to right,
+ * and the groups are added in a balanced binary tree over 64 slots (empty slots are 0); the scale is 1 / sqrtf(...)
+ * with IEEE division and square root (the reference uses the approximate rsqrtf, a difference of an ulp); the
+ * rotation angle is pos * (float) pow(base, -2j/n_rot) in fp32 and its cosine / sine are the double-precision ones
+ * rounded to fp32; products and sums are rounded separately (no fused multiply-add).
+ */
+static void prep_norm_rope(const float *src, const float *w, int D, int n_rot, float freq_base, float eps, int pos, float *dst) {
+    float part[64];
+    for (int i = 0; i < 64; ++i) {
+        part[i] = 0.0f;
+        if (4 * i < D) {
+            const float *a = src + 4 * i;
+            float s = a[0] * a[0];
+            s = s + a[1] * a[1];
+            s = s + a[2] * a[2];
+            s = s + a[3] * a[3];
+            part[i] = s;
+        }
+    }
+    for (int m = 1; m < 64; m <<= 1)
+        for (int i = 0; i < 64; i += 2 * m) part[i] = part[i] + part[i + m];
+    const float sc = 1.0f / sqrtf(part[0] / (float) D + eps);
+    for (int i = 0; i < D; ++i) {
+        float o = src[i] * sc;
+        if (w) o = o * w[i];
+        dst[i] = o;
+    }
+    const int half = n_rot / 2;
+    for (int j = 0; j < half; ++j) {
+        const float inv = (float) pow((double) freq_base, -2.0 * (double) j / (double) n_rot);
+        const float theta = (float) pos * inv;
+        const float c = (float) cos((double) theta), sn = (float) sin((double) theta);
+        const float x0 = dst[j], x1 = dst[j + half];
+        const float a0 = x0 * c, a1 = x1 * sn, b0 = x0 * sn, b1 = x1 * c;
+        dst[j] = a0 - a1;
+        dst[j + half] = b0 + b1;
+    }
+}
+
+int orc_attn_prep(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
+                  const int32_t *pos, float *q, float *gate, const orc_kv *c, int p0, int T, int Hq, int Hkv, int D,
+                  int n_rot, float freq_base, float eps, int ldq, int ldk, int ldv) {
+    if (!pos || D % 32 || D > 256 || n_rot % 8 || n_rot > D || c->D != D || c->Hkv != Hkv) return -1;
+    if (!ldq) ldq = Hq * 2 * D;
+    if (!ldk) ldk = Hkv * D;
+    if (!ldv) ldv = Hkv * D;
+    float *kr = (float *) malloc(sizeof(float) * (size_t) Hkv * D);
+    float *vr = (float *) malloc(sizeof(float) * (size_t) Hkv * D);
+    orc_kv one = *c;
+    for (int t = 0; t < T; ++t) {
+        for (int h = 0; h < Hq; ++h) {
+            const float *src = qg + (size_t) t * ldq + (size_t) h * 2 * D;
+            memcpy(gate + ((size_t) t * Hq + h) * D, src + D, sizeof(float) * D);
+            prep_norm_rope(src, q_norm, D, n_rot, freq_base, eps, pos[t], q + ((size_t) t * Hq + h) * D);
+        }
+        for (int h = 0; h < Hkv; ++h) {
+            prep_norm_rope(k + (size_t) t * ldk + (size_t) h * D, k_norm, D, n_rot, freq_base, eps, pos[t], kr + (size_t) h * D);
+            memcpy(vr + (size_t) h * D, v + (size_t) t * ldv + (size_t) h * D, sizeof(float) * D);
+        }
+        /* row t of the batch: its own page table (rtab[t]) and its own position */
+        const int32_t row = p0 < 0 ? pos[t] : p0 + t;
+        one.rtab = c->rtab ? c->rtab + t : NULL;
+        orc_kv_append_rows(&one, kr, vr, &row, 1);
+    }
+    free(kr);
+    free(vr);
+    return 0;
+}
+
 int orc_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -14,6 +14,9 @@
  *   orc_attn_rows                              : numpy float64 softmax(QK^T)V on the dequantized cache, n = 1,
  *       equal-V, dominant-logit, causality and shift-invariance closed forms.
  *   orc_gate                                   : g = 0 -> x0.5, sigma(g) + sigma(-g) = 1.
+ *   orc_attn_prep                              : numpy float64 restatement of norm * weight and the NEOX rotation (to a few
+ *       fp32 ulps); closed forms (position 0 rotates nothing, the rotation keeps pair norms, q . k after rope depends on
+ *       the position difference only, a constant head norms to w); KV rows == orc_kv_append_rows of the normed, roped k.
  * No function of this file is "parity unpinned".
  */
 #ifndef P1A_ORACLE_H
@@ -61,6 +64,12 @@ int orc_attn_rows(const orc_kv *c, const float *q, float *out, const float *gate
 void orc_gate(float *x, const float *g, size_t n);
 /* per-head RMS norm with unit weight, in place: x * rsqrt(mean(x^2) + eps) */
 void orc_rmsnorm_heads(float *x, size_t nheads, int D, float eps);
+/* attention-layer input prep (q | gate split, RMS norm * weight, NEOX rope, quantize-append): src/fast/fused.cuh:101-113.
+ * qg [T][ldq] (Hq heads of q | gate), k, v [T][ld] f32; q [T][Hq][D], gate [T][Hq*D] out; K / V rows written to c.
+ * ld* = 0: dense. q_norm / k_norm [D] may be NULL. Returns 0, or -1 for an unsupported shape. */
+int orc_attn_prep(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
+                  const int32_t *pos, float *q, float *gate, const orc_kv *c, int p0, int T, int Hq, int Hkv, int D,
+                  int n_rot, float freq_base, float eps, int ldq, int ldk, int ldv);
 int orc_num_threads(void);
 
 #ifdef __cplusplus

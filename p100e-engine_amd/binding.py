@@ -1,13 +1,13 @@
 """ctypes binding of include/p1a_attn.h. Function names follow the reference's C++ surface
 (src/fast/attn.cuh:34-70 of the reference tree): kv_append, kv_append_dev, attn_decode, attn_decode_dev,
-attn_decode_rows, attn_prefill."""
+attn_decode_rows, attn_prefill; attn_prep is src/fast/fused.cuh:101-113."""
 import ctypes
 import os
 
 KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
-    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_decode", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
+    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_decode", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_release", "p1a_last_error",
     "p1a_version",
 ]
@@ -47,6 +47,8 @@ def lib():
     L.p1a_kv_row_bytes.argtypes = [ctypes.c_uint32, i32, i32]
     L.p1a_kv_append.restype = i32
     L.p1a_kv_append.argtypes = [kvp, vp, vp, i32, vp, vp, i32, vp]
+    L.p1a_attn_prep.restype = i32
+    L.p1a_attn_prep.argtypes = [vp] * 8 + [kvp, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp]
     L.p1a_attn_decode.restype = i32
     L.p1a_attn_decode.argtypes = [vp, kvp, vp, vp, i32, i32, vp, vp, i32, i32, f32, vp]
     L.p1a_attn_prefill.restype = i32
@@ -161,6 +163,13 @@ def kv_append_rows(c, k, v, pos_rows, T):
     """Cache-write half of attn_prep in device-position mode (src/fast/fused.cuh:101-113): row t -> pos_rows[t] of
     its own sequence (c.rtab)."""
     _check(lib().p1a_kv_append(ctypes.byref(c.struct()), _ptr(k), _ptr(v), -1, None, _ptr(pos_rows), T, _stream()), "kv_append_rows")
+
+
+def attn_prep(qg, k, v, q_norm, k_norm, pos, q, gate, c, p0, T, Hq, n_rot, freq_base, eps, ldq=0, ldk=0, ldv=0):
+    """src/fast/fused.cuh:101-113: q | gate split, per-head RMS norm * weight, NEOX rope, quantizing KV write (p0 < 0:
+    cache row of token t = pos[t], its own page table)."""
+    _check(lib().p1a_attn_prep(_ptr(qg), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(pos), _ptr(q), _ptr(gate),
+                               ctypes.byref(c.struct()), p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, _stream()), "attn_prep")
 
 
 def attn_decode(q, c, out, T, p0, Hq, scale, gate=None):

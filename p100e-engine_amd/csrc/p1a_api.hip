@@ -107,6 +107,28 @@ int p1a_kv_append(const p1a_kv * c, const float * k, const float * v, int p0, co
     return launch_append(*c, k, v, p0, p0_dev, pos_rows, T, (hipStream_t) stream);
 }
 
+int p1a_attn_prep(const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
+                  const int32_t * pos, float * q, float * gate, const p1a_kv * c, int p0, int T, int Hq, int n_rot,
+                  float freq_base, float eps, int ldq, int ldk, int ldv, void * stream) {
+    if (!kv_ok(c, "p1a_attn_prep")) return P1A_E_ARG;
+    if (!qg || !k || !v || !pos || !q || !gate || T < 0 || Hq < 1) { set_error("p1a_attn_prep: null argument or bad T / Hq"); return P1A_E_ARG; }
+    if (T == 0) return P1A_OK;
+    const int D = c->D, Hkv = c->Hkv;
+    if (D > 256 || n_rot < 0 || n_rot % 8 || n_rot > D || T > 65535) {
+        set_error("p1a_attn_prep: unsupported shape (D=%d n_rot=%d T=%d): D <= 256, n_rot %% 8 == 0, n_rot <= D", D, n_rot, T);
+        return P1A_E_SHAPE;
+    }
+    if (!ldq) ldq = Hq * 2 * D;
+    if (!ldk) ldk = Hkv * D;
+    if (!ldv) ldv = Hkv * D;
+    const uintptr_t al = (uintptr_t) qg | (uintptr_t) k | (uintptr_t) v | (uintptr_t) q | (uintptr_t) gate | (uintptr_t) q_norm | (uintptr_t) k_norm;
+    if ((al & 15) || ((ldq | ldk | ldv) & 3) || ldq < Hq * 2 * D || ldk < Hkv * D || ldv < Hkv * D) {
+        set_error("p1a_attn_prep: pointers must be 16-byte aligned, row strides multiples of 4 floats and at least one row");
+        return P1A_E_SHAPE;
+    }
+    return launch_prep(*c, qg, k, v, q_norm, k_norm, pos, q, gate, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, (hipStream_t) stream);
+}
+
 int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float * gate, int T, int p0,
                     const int32_t * p0_dev, const int32_t * pos_rows, int rows_per_seq, int Hq, float scale,
                     void * stream) {

@@ -4,6 +4,9 @@
 // and the sum separately, and uses IEEE division for amax / 127 and 1 / d.
 // Mapping: one lane owns 4 consecutive values (one 16-byte load for K, one for V), 8 lanes own a 32-value block and
 // reduce over it with three xor-shuffles; a 256-thread workgroup covers 1024 values of one position row.
+// The attention-layer input prep (q | gate split, per-head RMS norm * weight, NEOX rope, the same quantizing write) lives
+// here too: its K codes depend on the last bit of the normed, rotated values, so it keeps a fixed operation order under
+// the same no-contraction rule.
 #include "p1a_common.hpp"
 
 #pragma clang fp contract(off)
@@ -107,6 +110,101 @@ __global__ void __launch_bounds__(256) append_k(const float * __restrict__ k, co
     }
 }
 
+// ---- attention-layer input prep: one wave per (head, token); lane i owns dims 4 i .. 4 i + 3 of the head ----
+// Replaces the front half of the reference's attn_prep kernel (src/fast/fused.cu:512-573). Heads b < Hq are q heads
+// (gate copy, norm, rope, store), Hq <= b < Hq + Hkv k heads (norm, rope, quantizing write), the rest v heads (write).
+// Operation order (the CPU oracle keeps the same one, so K codes compare bit for bit): the squares of a lane's 4 values
+// are added left to right, the 64 lane sums in a butterfly (a balanced binary tree); scale = 1 / sqrtf(ss / D + eps)
+// with IEEE division and square root; angle = pos * (float) pow(base, -2 j / n_rot) in fp32, cosine and sine in double
+// precision rounded to fp32; every product and sum rounded on its own.
+template <uint32_t KT>
+__global__ void __launch_bounds__(64) prep_k(const float * __restrict__ qg, const float * __restrict__ k,
+                                             const float * __restrict__ v, const float * __restrict__ qn,
+                                             const float * __restrict__ kn, const int32_t * __restrict__ pos,
+                                             float * __restrict__ q, float * __restrict__ gate, char * kc, char * vc, int p0,
+                                             int Hq, int Hkv, int D, int n_rot, float freq_base, float eps, int ldq, int ldk,
+                                             int ldv, kv_view pg) {
+    const int t = blockIdx.y, b = blockIdx.x, i = threadIdx.x;
+    const bool live = 4 * i < D;                               // dead lanes form whole 8-lane groups (D % 32 == 0)
+    const int row = p0 < 0 ? pos[t] : p0 + t;                  // cache position of token t (src/fast/fused.cu:520)
+    const size_t o = kv_off_tab(pg, kv_tab(pg, t), row);
+    const int nb = D / 32, blk = i >> 3, j8 = i & 7;
+    auto write_head = [&](char * cache, int h, float4 x) {
+        if constexpr (KT == P1A_KV_F16) {
+            if (live) reinterpret_cast<h4 *>(cache + o + (size_t) h * D * 2)[i] = h4{(half_t) x.x, (half_t) x.y, (half_t) x.z, (half_t) x.w};
+        } else if constexpr (KT == P1A_KV_Q8_0) {
+            if (live) q8_block(x, j8, cache + o + (size_t) h * nb * 34, blk, nb);
+            else xor8_max(0.f);
+        } else {
+            if (live) q4_block(x, j8, cache + o + ((size_t) h * nb + blk) * 18);
+        }
+    };
+    if (b >= Hq + Hkv) {                                       // v head: the plain quantizing write
+        const int h = b - Hq - Hkv;
+        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) x = reinterpret_cast<const float4 *>(v + (size_t) t * ldv + (size_t) h * D)[i];
+        write_head(vc, h, x);
+        return;
+    }
+    const bool isq = b < Hq;
+    const int h = isq ? b : b - Hq;
+    const float * src = isq ? qg + (size_t) t * ldq + (size_t) h * 2 * D : k + (size_t) t * ldk + (size_t) h * D;
+    const float * w = isq ? qn : kn;
+    float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (live) {
+        a = reinterpret_cast<const float4 *>(src)[i];
+        if (isq) reinterpret_cast<float4 *>(gate + ((size_t) t * Hq + h) * D)[i] = reinterpret_cast<const float4 *>(src + D)[i];
+    }
+    float ss = a.x * a.x;
+    ss = ss + a.y * a.y;
+    ss = ss + a.z * a.z;
+    ss = ss + a.w * a.w;
+#pragma unroll
+    for (int m = 1; m < 64; m <<= 1) ss = ss + __shfl_xor(ss, m);
+    const float sc = 1.0f / sqrtf(ss / (float) D + eps);
+    float x[4] = {a.x * sc, a.y * sc, a.z * sc, a.w * sc};
+    if (w && live) {
+        const float4 ww = reinterpret_cast<const float4 *>(w)[i];
+        x[0] = x[0] * ww.x; x[1] = x[1] * ww.y; x[2] = x[2] * ww.z; x[3] = x[3] * ww.w;
+    }
+    // NEOX rope: dims d < n_rot / 2 pair with d + n_rot / 2, which lane i + n_rot / 8 holds in the same slot
+    const int half = n_rot >> 1, hl = half >> 2;
+    const bool lo = i < hl, rot = i < 2 * hl;
+    const int partner = lo ? i + hl : i - hl;
+    const float posf = (float) pos[t];
+    // the angle tables of the head: pair j is computed once, by lane j & 63 (slot j >> 6), and handed round by shuffle
+    float tc[2] = {1.f, 1.f}, tsn[2] = {0.f, 0.f};
+#pragma unroll
+    for (int sl = 0; sl < 2; ++sl) {
+        const int jj = i + 64 * sl;
+        if (jj < half) {
+            const float inv = (float) pow((double) freq_base, -2.0 * (double) jj / (double) n_rot);
+            const float theta = posf * inv;
+            tc[sl] = (float) cos((double) theta);
+            tsn[sl] = (float) sin((double) theta);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const float other = __shfl(x[e], rot ? partner : i);
+        const int jj = rot ? 4 * (lo ? i : i - hl) + e : 0;
+        const float c0 = __shfl(tc[0], jj & 63), c1 = __shfl(tc[1], jj & 63);
+        const float s0 = __shfl(tsn[0], jj & 63), s1 = __shfl(tsn[1], jj & 63);
+        if (rot) {
+            const float c = jj < 64 ? c0 : c1, sn = jj < 64 ? s0 : s1;
+            const float x0 = lo ? x[e] : other, x1 = lo ? other : x[e];
+            const float p0_ = x0 * (lo ? c : sn), p1_ = x1 * (lo ? sn : c);
+            x[e] = lo ? p0_ - p1_ : p0_ + p1_;
+        }
+    }
+    const float4 r = make_float4(x[0], x[1], x[2], x[3]);
+    if (isq) {
+        if (live) reinterpret_cast<float4 *>(q + ((size_t) t * Hq + h) * D)[i] = r;
+    } else {
+        write_head(kc, h, r);
+    }
+}
+
 }   // namespace
 
 int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, const int32_t * p0_dev,
@@ -118,6 +216,21 @@ int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, co
     if (c.type == P1A_KV_F16) append_k<P1A_KV_F16><<<grid, 256, 0, s>>>(k, v, kc, vc, p0, p0_dev, pos_rows, c.Hkv, c.D, pg);
     else if (c.type == P1A_KV_Q8_0) append_k<P1A_KV_Q8_0><<<grid, 256, 0, s>>>(k, v, kc, vc, p0, p0_dev, pos_rows, c.Hkv, c.D, pg);
     else append_k<P1A_KV_Q4_0><<<grid, 256, 0, s>>>(k, v, kc, vc, p0, p0_dev, pos_rows, c.Hkv, c.D, pg);
+    return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
+}
+
+int launch_prep(const p1a_kv & c, const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
+                const int32_t * pos, float * q, float * gate, int p0, int T, int Hq, int n_rot, float freq_base, float eps,
+                int ldq, int ldk, int ldv, hipStream_t s) {
+    const kv_view pg = view_of(c);
+    const dim3 grid(Hq + 2 * c.Hkv, T);
+    char * kc = (char *) c.k, * vc = (char *) c.v;
+#define P1A_PREP(KT_) prep_k<KT_><<<grid, 64, 0, s>>>(qg, k, v, q_norm, k_norm, pos, q, gate, kc, vc, p0, Hq, c.Hkv, c.D, n_rot, \
+                                                      freq_base, eps, ldq, ldk, ldv, pg)
+    if (c.type == P1A_KV_F16) P1A_PREP(P1A_KV_F16);
+    else if (c.type == P1A_KV_Q8_0) P1A_PREP(P1A_KV_Q8_0);
+    else P1A_PREP(P1A_KV_Q4_0);
+#undef P1A_PREP
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 

@@ -633,6 +633,9 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
     const int d = blockIdx.y * 32 + q4 * 4;
     const float * ml = part_ml + row * NS * 2;
     constexpr int CH = 8;                                     // splits of a slice fetched together
+    // the gate depends on nothing here: its load rides along with the first batch of partials
+    f4 gt = {0.f, 0.f, 0.f, 0.f};
+    if (gate && sl == 0) gt = *reinterpret_cast<const f4 *>(gate + row * D + d);
     float M = NEG_INF;
     for (int s = tid; s < NS; s += 64) M = fmaxf(M, ml[2 * s]);
     // the partials do not depend on M: request the first batch before the maximum is reduced
@@ -682,7 +685,6 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
         for (int k = 1; k < 8; ++k) { n += sacc[k][q4]; dn += sden[k]; }
         f4 r = {n[0] / dn, n[1] / dn, n[2] / dn, n[3] / dn};
         if (gate) {
-            const f4 gt = *reinterpret_cast<const f4 *>(gate + row * D + d);
 #pragma unroll
             for (int x = 0; x < 4; ++x) r[x] *= 1.0f / (1.0f + expf(-gt[x]));
         }

@@ -44,6 +44,8 @@ def lib():
                                     ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_int]
         L.orc_gate.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
         L.orc_rmsnorm_heads.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_float]
+        L.orc_attn_prep.argtypes = [ctypes.c_void_p] * 8 + [ctypes.POINTER(orc_kv)] + [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 3
+        L.orc_attn_prep.restype = ctypes.c_int
         L.orc_num_threads.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -144,3 +146,20 @@ def rmsnorm_heads(x, D, eps=1e-6):
     x = np.ascontiguousarray(x, np.float32).copy()
     lib().orc_rmsnorm_heads(_p(x), x.size // D, D, eps)
     return x
+
+
+def attn_prep(c, qg, k, v, q_norm, k_norm, pos, p0, Hq, n_rot, freq_base, eps=1e-6):
+    """q | gate split, norm, rope, quantize-append: returns (q, gate); K / V rows are written into c."""
+    qg = np.ascontiguousarray(qg, np.float32)
+    k = np.ascontiguousarray(k, np.float32)
+    v = np.ascontiguousarray(v, np.float32)
+    pos = np.ascontiguousarray(pos, np.int32)
+    T = len(pos)
+    q = np.zeros((T, Hq, c.D), np.float32)
+    gate = np.zeros((T, Hq * c.D), np.float32)
+    qn = None if q_norm is None else np.ascontiguousarray(q_norm, np.float32)
+    kn = None if k_norm is None else np.ascontiguousarray(k_norm, np.float32)
+    rc = lib().orc_attn_prep(_p(qg), _p(k), _p(v), _p(qn), _p(kn), _p(pos), _p(q), _p(gate), ctypes.byref(c.struct()), p0, T, Hq,
+                             c.Hkv, c.D, n_rot, freq_base, eps, 0, 0, 0)
+    assert rc == 0, rc
+    return q, gate

@@ -132,6 +132,34 @@ static void test_type(uint32_t type, hipStream_t s) {
         auto a = bytes_of(o1, (size_t) T * Hq * D * 4), b = bytes_of(o2, (size_t) T * Hq * D * 4);
         check("attn_prefill T=200 p0=1300 paged vs contiguous", a1 && a2 && !memcmp(a.data(), b.data(), a.size()));
     }
+    {   // attn_prep: host positions on the contiguous cache vs device positions through the page table (one sequence)
+        const int sq = 2, T = 4, p0 = len[sq] - T, n_rot = 64;
+        float * qg = dev_rand((size_t) T * Hq * 2 * D, 1.0f), * kk = dev_rand((size_t) T * Hkv * D, 1.0f), * vv = dev_rand((size_t) T * Hkv * D, 1.0f);
+        float * wn = dev_rand((size_t) D, 1.0f), * g1, * g2;
+        CK(hipMalloc(&g1, (size_t) T * Hq * D * 4)); CK(hipMalloc(&g2, (size_t) T * Hq * D * 4));
+        int32_t * dpos, * drt; CK(hipMalloc(&dpos, 64)); CK(hipMalloc(&drt, 64));
+        std::vector<int32_t> hp(T), hr(T, sq * MAXP);
+        for (int t = 0; t < T; ++t) hp[t] = p0 + t;
+        CK(hipMemcpy(dpos, hp.data(), T * 4, hipMemcpyHostToDevice)); CK(hipMemcpy(drt, hr.data(), T * 4, hipMemcpyHostToDevice));
+        F::kv_cache pc = paged(0);
+        pc.pt = dtab; pc.rtab = drt;
+        const bool a1 = F::attn_prep(qg, kk, vv, wn, wn, dpos, o1, g1, cc[sq], p0, T, Hq, Hkv, D, n_rot, 1e7f, 1e-6f, s);
+        const bool a2 = F::attn_prep(qg, kk, vv, wn, wn, dpos, o2, g2, pc, -1, T, Hq, Hkv, D, n_rot, 1e7f, 1e-6f, s);
+        CK(hipStreamSynchronize(s));
+        bool ok = a1 && a2;
+        auto qa = bytes_of(o1, (size_t) T * Hq * D * 4), qb = bytes_of(o2, (size_t) T * Hq * D * 4);
+        auto ga = bytes_of(g1, (size_t) T * Hq * D * 4), gb = bytes_of(g2, (size_t) T * Hq * D * 4);
+        ok = ok && !memcmp(qa.data(), qb.data(), qa.size()) && !memcmp(ga.data(), gb.data(), ga.size());
+        auto hpool = bytes_of(pool, (size_t) NP * pstride);
+        auto hk = bytes_of(cc[sq].k, (size_t) len[sq] * rowb), hv = bytes_of(cc[sq].v, (size_t) len[sq] * rowb);
+        for (int p = p0; p < p0 + T; ++p) {
+            const size_t o = (size_t) tabs[(size_t) sq * MAXP + (p >> PSH)] * pstride + (size_t) 2 * PS * rowb + (size_t) (p & (PS - 1)) * rowb;
+            ok = ok && !memcmp(hk.data() + (size_t) p * rowb, hpool.data() + o, rowb);
+            ok = ok && !memcmp(hv.data() + (size_t) p * rowb, hpool.data() + o + PS * rowb, rowb);
+        }
+        check("attn_prep host positions vs device positions + page table", ok);
+        CK(hipFree(qg)); CK(hipFree(kk)); CK(hipFree(vv)); CK(hipFree(wn)); CK(hipFree(g1)); CK(hipFree(g2)); CK(hipFree(dpos)); CK(hipFree(drt));
+    }
     {   // a refusal launches nothing and leaves out untouched
         CK(hipMemset(o1, 0x5a, 4096));
         const bool r = F::attn_decode(q, cc[0], o1, 1, 10, Hq + 1, scale, s);

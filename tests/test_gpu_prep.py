@@ -1,0 +1,112 @@
+"""attn_prep on the GPU (through the C ABI) vs the oracle: gate and KV bytes must match bit for bit, q to the last
+bit as well (both sides keep one operation order); then the prepared cache and q drive a decode."""
+import numpy as np
+import pytest
+import torch
+
+import _inputs as I
+import _oracle as O
+from _gpu import check, dev
+
+pytestmark = pytest.mark.gpu
+TYPES = [O.KV_F16, O.KV_Q8_0, O.KV_Q4_0]
+
+
+def make(seed, T, Hq, Hkv, D):
+    g = I.rng(seed)
+    qg = I.normal(g, (T, Hq, 2 * D))
+    k = I.normal(g, (T, Hkv, D)) * 1.3
+    v = I.normal(g, (T, Hkv, D))
+    qn = (1.0 + 0.1 * I.normal(g, (D,))).astype(np.float32)
+    kn = (1.0 + 0.1 * I.normal(g, (D,))).astype(np.float32)
+    return qg, k, v, qn, kn
+
+
+def ulp_diff(a, b):
+    ia = a.view(np.int32).astype(np.int64)
+    ib = b.view(np.int32).astype(np.int64)
+    ia = np.where(ia < 0, -(ia & 0x7fffffff), ia)
+    ib = np.where(ib < 0, -(ib & 0x7fffffff), ib)
+    return np.abs(ia - ib)
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,n_rot", [(24, 4, 256, 64), (4, 1, 64, 64), (8, 2, 128, 32)])
+def test_host_position_contiguous(p1a, kv_type, Hq, Hkv, D, n_rot):
+    T, p0, n_ctx, base, eps = 7, 9, 32, 1e7, 1e-6
+    qg, k, v, qn, kn = make(D + n_rot, T, Hq, Hkv, D)
+    pos = (p0 + np.arange(T)).astype(np.int32)
+    host = O.HostKV.contiguous(kv_type, n_ctx, Hkv, D)
+    q_ref, gate_ref = O.attn_prep(host, qg, k, v, qn, kn, pos, p0, Hq, n_rot, base, eps)
+    c = p1a.KVCache.contiguous(kv_type, n_ctx, Hkv, D)
+    q = torch.zeros((T, Hq, D), device="cuda")
+    gate = torch.zeros((T, Hq * D), device="cuda")
+    p1a.attn_prep(dev(qg), dev(k), dev(v), dev(qn), dev(kn), dev(pos), q, gate, c, p0, T, Hq, n_rot, base, eps)
+    torch.cuda.synchronize()
+    assert np.array_equal(gate.cpu().numpy(), gate_ref)
+    qd = q.cpu().numpy()
+    assert ulp_diff(qd, q_ref).max() <= 1, ulp_diff(qd, q_ref).max()      # cos / sin: two double libraries, rounded to fp32
+    assert np.mean(qd.view(np.int32) == q_ref.view(np.int32)) > 0.999
+    assert np.array_equal(c._keep[1].cpu().numpy(), host.v)
+    kd = c._keep[0].cpu().numpy()
+    assert np.mean(kd == host.k) > 0.999                                   # (a last-bit difference may move a code)
+    if not np.array_equal(kd, host.k):
+        bad = np.nonzero(kd != host.k)[0]
+        assert len(bad) <= 4, len(bad)
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_device_positions_paged_rows_then_decode(p1a, kv_type):
+    """rows of four sequences, each at its own position through its own page table (p0 < 0), strided inputs; then the
+    prepared q / gate / cache drive attn_decode_rows and must give the oracle's attention"""
+    Hq, Hkv, D, n_rot, base, eps, psh = 12, 2, 256, 64, 1e7, 1e-6, 4
+    lens = [40, 17, 63, 5]
+    T = len(lens)
+    max_pages, n_pages = 5, 24
+    g = I.rng(77)
+    table = g.permutation(n_pages)[: T * max_pages].astype(np.int32)
+    rtab = (np.arange(T) * max_pages).astype(np.int32)
+    host = O.HostKV.paged(kv_type, Hkv, D, psh, n_pages, table, max_pages).view(rtab=rtab)
+    dtab, drt = dev(table), dev(rtab)
+    dc = p1a.KVCache.paged(kv_type, Hkv, D, psh, n_pages, dtab, max_pages).with_rows(drt)
+    # history: every sequence gets lens[s] - 1 earlier rows through the plain append (same bytes on both sides)
+    for s, n in enumerate(lens):
+        if n > 1:
+            _, kh, vh, _ = I.qkv(900 + s, n - 1, 1, Hq, Hkv, D)
+            O.kv_append_rows(host.view(rtab=np.full(n - 1, s * max_pages, np.int32)), kh, vh, np.arange(n - 1))
+            p1a.kv_append(dc.slot(s, max_pages), dev(kh), dev(vh), 0, n - 1)
+    qg, k, v, qn, kn = make(5, T, Hq, Hkv, D)
+    pos = np.array([n - 1 for n in lens], np.int32)
+    # strided inputs: rows carry padding, as slices of a concatenated projection output do
+    ldq, ldk, ldv = Hq * 2 * D + 8, Hkv * D + 4, Hkv * D + 12
+    def strided(a, ld):
+        buf = np.full((T, ld), 7.0, np.float32)
+        buf[:, : a[0].size] = a.reshape(T, -1)
+        return buf
+    q_ref, gate_ref = O.attn_prep(host, qg, k, v, qn, kn, pos, -1, Hq, n_rot, base, eps)
+    q = torch.zeros((T, Hq, D), device="cuda")
+    gate = torch.zeros((T, Hq * D), device="cuda")
+    dpos = dev(pos)
+    p1a.attn_prep(dev(strided(qg, ldq)), dev(strided(k, ldk)), dev(strided(v, ldv)), dev(qn), dev(kn), dpos, q, gate, dc, -1, T, Hq,
+                  n_rot, base, eps, ldq=ldq, ldk=ldk, ldv=ldv)
+    torch.cuda.synchronize()
+    assert np.array_equal(gate.cpu().numpy(), gate_ref)
+    assert ulp_diff(q.cpu().numpy(), q_ref).max() <= 1
+    out = torch.zeros((T, Hq, D), device="cuda")
+    p1a.attn_decode_rows(q, dc, out, T, dpos, Hq, 1 / 16, gate=gate)
+    torch.cuda.synchronize()
+    ref = O.attn_rows(host, q_ref, pos, Hq, 1 / 16, gate=gate_ref)
+    check(out.cpu().numpy(), ref, f"prep -> decode_rows type {kv_type}")
+
+
+def test_refusals(p1a):
+    c = p1a.KVCache.contiguous(O.KV_Q8_0, 8, 2, 256)
+    z = torch.zeros(4 * 2 * 256 * 2, device="cuda")
+    pos = torch.zeros(1, dtype=torch.int32, device="cuda")
+    with pytest.raises(p1a.P1AError):       # n_rot not a multiple of 8
+        p1a.attn_prep(z, z, z, None, None, pos, z, z, c, 0, 1, 4, 12, 1e7, 1e-6)
+    with pytest.raises(p1a.P1AError):       # no positions
+        p1a.attn_prep(z, z, z, None, None, None, z, z, c, 0, 1, 4, 64, 1e7, 1e-6)
+    with pytest.raises(p1a.P1AError):       # row stride shorter than a row
+        p1a.attn_prep(z, z, z, None, None, pos, z, z, c, 0, 1, 4, 64, 1e7, 1e-6, ldq=64)
+    torch.cuda.synchronize()

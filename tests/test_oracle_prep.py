@@ -1,0 +1,113 @@
+"""Pins the oracle's attn_prep (a restatement of src/fast/fused.cu:512-573 of the reference: q | gate split, per-head
+RMS norm * weight, NEOX rope on the first n_rot dims, quantize-append) against numpy float64 and closed forms."""
+import numpy as np
+import pytest
+
+import _oracle as O
+import _inputs as I
+
+TYPES = [O.KV_F16, O.KV_Q8_0, O.KV_Q4_0]
+
+
+def np_norm_rope(x, w, n_rot, base, eps, pos):
+    """float64 textbook: x * rsqrt(mean(x^2) + eps) * w, then rotate pairs (j, j + n_rot/2) by pos * base^(-2j/n_rot)"""
+    x = x.astype(np.float64)
+    y = x / np.sqrt((x * x).mean() + eps)
+    if w is not None:
+        y = y * w.astype(np.float64)
+    half = n_rot // 2
+    j = np.arange(half)
+    th = pos * base ** (-2.0 * j / n_rot)
+    c, s = np.cos(th), np.sin(th)
+    x0, x1 = y[:half].copy(), y[half:n_rot].copy()
+    y[:half] = x0 * c - x1 * s
+    y[half:n_rot] = x0 * s + x1 * c
+    return y
+
+
+def make(seed, T, Hq, Hkv, D):
+    g = I.rng(seed)
+    qg = I.normal(g, (T, Hq, 2 * D))
+    k = I.normal(g, (T, Hkv, D))
+    v = I.normal(g, (T, Hkv, D))
+    qn = (1.0 + 0.1 * I.normal(g, (D,))).astype(np.float32)
+    kn = (1.0 + 0.1 * I.normal(g, (D,))).astype(np.float32)
+    return qg, k, v, qn, kn
+
+
+@pytest.mark.parametrize("Hq,Hkv,D,n_rot", [(24, 4, 256, 64), (4, 1, 64, 64), (8, 2, 128, 32)])
+def test_against_numpy_float64(Hq, Hkv, D, n_rot):
+    T, base, eps = 5, 1e7, 1e-6
+    qg, k, v, qn, kn = make(3, T, Hq, Hkv, D)
+    pos = np.array([0, 1, 17, 4000, 65535], np.int32)
+    c = O.HostKV.contiguous(O.KV_F16, 70000, Hkv, D)
+    q, gate = O.attn_prep(c, qg, k, v, qn, kn, pos, -1, Hq, n_rot, base, eps)
+    assert np.array_equal(gate.reshape(T, Hq, D), qg[:, :, D:])                 # the gate is a plain copy
+    for t in range(T):
+        for h in range(Hq):
+            ref = np_norm_rope(qg[t, h, :D], qn, n_rot, base, eps, float(pos[t]))
+            # fp32 angle: pos * inv_freq carries up to pos * 2^-24 of absolute angle error at the largest positions
+            tol = 4e-6 + 2.0 * pos[t] * 2.0 ** -24
+            assert np.max(np.abs(q[t, h] - ref)) < tol * max(1.0, np.abs(ref).max()), (t, h)
+        for h in range(Hkv):
+            ref = np_norm_rope(k[t, h], kn, n_rot, base, eps, float(pos[t]))
+            got = O.kv_read_head(c, 0, 0, int(pos[t]), h)                       # f16 cache: half precision of the roped k
+            assert np.max(np.abs(got - ref)) < 2e-3 * max(1.0, np.abs(ref).max())
+            assert np.array_equal(O.kv_read_head(c, 1, 0, int(pos[t]), h), v[t, h].astype(np.float16).astype(np.float32))
+
+
+def test_closed_forms():
+    Hq, Hkv, D, n_rot, base = 2, 1, 64, 64, 1e4
+    qg, k, v, qn, kn = make(8, 3, Hq, Hkv, D)
+    c = O.HostKV.contiguous(O.KV_F16, 64, Hkv, D)
+    # position 0 rotates nothing: q is the plain norm
+    q0, _ = O.attn_prep(c, qg, k, v, None, None, np.zeros(3, np.int32), 0, Hq, n_rot, base)
+    ref = O.rmsnorm_heads(qg[:, :, :D].copy(), D)
+    assert np.max(np.abs(q0 - ref)) < 2e-6
+    # a constant head norms to +-1 * w (eps aside)
+    qc = np.full((1, Hq, 2 * D), -3.0, np.float32)
+    q1, _ = O.attn_prep(c, qc, k[:1], v[:1], qn, None, np.zeros(1, np.int32), 0, Hq, n_rot, base, eps=0.0)
+    assert np.allclose(q1[0, 0], -qn, rtol=0, atol=2e-7)
+    # the rotation keeps the norm of every pair, and q . k after rope depends on the position difference only
+    pa = np.array([5, 105, 1005], np.int32)
+    kk = np.repeat(k[:1], 3, 0)
+    qq = np.repeat(qg[:1], 3, 0)
+    ca = O.HostKV.contiguous(O.KV_F16, 2048, Hkv, D)
+    qa, _ = O.attn_prep(ca, qq, kk, v, None, None, pa, -1, Hq, n_rot, base)
+    qb, _ = O.attn_prep(ca, qq, kk, v, None, None, pa + 7, -1, Hq, n_rot, base)
+    half = n_rot // 2
+    n0 = qa[:, :, :half] ** 2 + qa[:, :, half:n_rot] ** 2
+    n1 = q0[:1, :, :half] ** 2 + q0[:1, :, half:n_rot] ** 2
+    assert np.allclose(n0, np.repeat(n1, 3, 0), rtol=2e-5, atol=1e-6)
+    # <rope(x, p + 7), rope(y, p)> is the same for every p: use q head 0 as x, q head 1 as y
+    dots = [(qb[i, 0].astype(np.float64) * qa[i, 1].astype(np.float64)).sum() for i in range(3)]
+    assert max(dots) - min(dots) < 2e-3 * max(1.0, abs(dots[0]))
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_kv_rows_are_the_append_of_the_roped_k(kv_type):
+    """device-position mode, per-row page tables: the K / V bytes equal a plain append of the normed, roped k"""
+    Hq, Hkv, D, n_rot, base, psh = 8, 2, 128, 64, 1e7, 4
+    T = 4
+    qg, k, v, qn, kn = make(11, T, Hq, Hkv, D)
+    max_pages, n_pages = 8, 40
+    g = I.rng(5)
+    table = g.permutation(n_pages)[: T * max_pages].astype(np.int32)
+    rtab = (np.arange(T) * max_pages).astype(np.int32)
+    pos = np.array([0, 33, 100, 127], np.int32)
+    c1 = O.HostKV.paged(kv_type, Hkv, D, psh, n_pages, table, max_pages).view(rtab=rtab)
+    c1.pool = None
+    O.attn_prep(c1, qg, k, v, qn, kn, pos, -1, Hq, n_rot, base)
+    # reference chain: norm + rope through the q path of the same function (heads of k fed as "q | gate" slices)
+    kq = np.concatenate([k, np.zeros_like(k)], axis=2)
+    cf = O.HostKV.contiguous(O.KV_F16, 128, Hkv, D)
+    kr, _ = O.attn_prep(cf, kq, k, v, kn, None, pos, -1, Hkv, n_rot, base)
+    c2 = O.HostKV.paged(kv_type, Hkv, D, psh, n_pages, table, max_pages).view(rtab=rtab)
+    O.kv_append_rows(c2, kr, v, pos)
+    assert np.array_equal(c1.k, c2.k) and np.array_equal(c1.v, c2.v)
+    # host-position mode writes rows p0 + t of ONE table while the angle still follows pos[t]
+    c3 = O.HostKV.contiguous(kv_type, 16, Hkv, D)
+    c4 = O.HostKV.contiguous(kv_type, 16, Hkv, D)
+    O.attn_prep(c3, qg, k, v, qn, kn, pos, 3, Hq, n_rot, base)
+    O.kv_append_rows(c4, kr, v, 3 + np.arange(T))
+    assert np.array_equal(c3.k, c4.k) and np.array_equal(c3.v, c4.v)
