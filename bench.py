@@ -191,6 +191,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB elementwise copy kernel (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--prefill-only", action="store_true",
+                    help="run only the chunked-prefill configuration (T = 4096 after 28672 tokens, q8_0) a few times and print its "
+                         "time: a short program for rocprofv3 counter passes over prefill_k")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU only (no collectives are part of it); run with --gpus 1", file=sys.stderr)
@@ -203,6 +206,17 @@ def main():
     p1a.lib()
     Hq, Hkv, D, psh, n_ctx = 24, 4, 256, 8, 32768
     scale = 1.0 / 16.0
+    if args.prefill_only:
+        p0, T = 28672, 4096
+        kvp, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, p0 + T, 1, seed=21)
+        c = kvp.slot(0, ppseq)
+        qp = torch.randn((T, Hq, D), device="cuda").half().float()
+        gp = torch.randn((T, Hq * D), device="cuda")
+        op = torch.empty((T, Hq, D), device="cuda")
+        sec = time_eager(torch, lambda: p1a.attn_prefill(qp, c, op, T, p0, Hq, scale, gate=gp), reps=3, warmup=1)
+        flop = 4.0 * D * Hq * (p0 * T + T * (T + 1) / 2)
+        print(json.dumps({"prefill_T4096_p28672_q8_0_ms": round(sec * 1e3, 4), "TFLOPs": round(flop / sec / 1e12, 1)}))
+        return
     rowb = p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
     step_bytes = 2 * n_ctx * rowb                                          # K + V of the visible positions
     n_pools = 8                                                            # 8 x 71 MB > 256 MB Infinity Cache
