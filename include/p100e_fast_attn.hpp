@@ -89,6 +89,13 @@ inline bool attn_prep(const float * qg, const float * k, const float * v, const 
     return p1a_attn_prep(qg, k, v, q_norm, k_norm, pos, q, gate, &p, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, s) == P1A_OK;
 }
 
+// src/fast/fused.cuh:91-98
+enum ew_op : int { EW_SILU_MUL = 0, EW_SIGMOID_MUL = 1 };
+inline bool ew_quant(ew_op op, const float * a, const float * b, float * y, void * qbuf, int T, int n, hipStream_t s,
+                     int lda = 0, int ldb = 0) {
+    return p1a_ew_quant((int) op, a, b, y, qbuf, T, n, lda, ldb, s) == P1A_OK;
+}
+
 // src/fast/attn.cuh:39-44. false = nothing launched, out untouched.
 inline bool attn_decode(const float * q, const kv_cache & c, float * out, int T, int p0, int Hq, float scale,
                         hipStream_t s, const float * gate = nullptr) {
@@ -96,19 +103,21 @@ inline bool attn_decode(const float * q, const kv_cache & c, float * out, int T,
     return p1a_attn_decode(q, &p, out, gate, T, p0, nullptr, nullptr, 0, Hq, scale, s) == P1A_OK;
 }
 // src/fast/attn.cuh:59-60 (max_n is accepted for source compatibility: the grid never depends on the depth)
+// (qbuf: also emit the a16 activation buffer of the gated rows, i.e. the ew_quant(EW_SIGMOID_MUL) that follows in the engine)
 inline bool attn_decode_dev(const float * q, const kv_cache & c, float * out, int T, const int32_t * p0_dev, int max_n,
-                            int Hq, float scale, hipStream_t s, const float * gate = nullptr) {
+                            int Hq, float scale, hipStream_t s, const float * gate = nullptr, void * qbuf = nullptr) {
     (void) max_n;
     const p1a_kv p = detail::pod(c);
-    return p1a_attn_decode(q, &p, out, gate, T, 0, p0_dev, nullptr, 0, Hq, scale, s) == P1A_OK;
+    return p1a_attn_decode_a16(q, &p, out, gate, qbuf, T, 0, p0_dev, nullptr, 0, Hq, scale, s) == P1A_OK;
 }
 // src/fast/attn.cuh:61-66
 constexpr int ATTN_MAX_ROWS = P1A_MAX_ROWS;
 inline bool attn_decode_rows(const float * q, const kv_cache & c, float * out, int T, const int32_t * pos, int Hq,
-                             float scale, hipStream_t s, const float * gate = nullptr, int rows_per_seq = 1) {
+                             float scale, hipStream_t s, const float * gate = nullptr, int rows_per_seq = 1,
+                             void * qbuf = nullptr) {
     if (!pos) return false;
     const p1a_kv p = detail::pod(c);
-    return p1a_attn_decode(q, &p, out, gate, T, 0, nullptr, pos, rows_per_seq, Hq, scale, s) == P1A_OK;
+    return p1a_attn_decode_a16(q, &p, out, gate, qbuf, T, 0, nullptr, pos, rows_per_seq, Hq, scale, s) == P1A_OK;
 }
 // src/fast/attn_dec2.cuh:17-20
 inline bool attn_decode2(const float * q, const kv_cache & c, float * out, int T, int p0, const int32_t * p0_dev, int Hq,

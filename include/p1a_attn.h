@@ -112,6 +112,25 @@ int p1a_attn_decode(const float *q, const p1a_kv *c, float *out, const float *ga
                     void *stream);
 
 /*
+ * The same call that also emits the a16 activation buffer of the (gated) output rows, the input format of the engine's
+ * quantized output-projection matvec: qbuf holds p1a_a16_bytes(T, Hq*D) bytes - per row and 32-value group 16 half2 of
+ * value / amax (the engine's slot order), then per row and group one half2 (amax, sum of the scaled values). qbuf ==
+ * NULL is p1a_attn_decode. Replaces attn_decode* followed by ew_quant(EW_SIGMOID_MUL, ...) at the fused decode call
+ * site (src/tp_model.cu:1388-1397; layout src/fast/a16q.cuh:1-10, arithmetic :21-45 = src/fast/matvec_a16.cu:29-100).
+ */
+int p1a_attn_decode_a16(const float *q, const p1a_kv *c, float *out, const float *gate, void *qbuf, int T, int p0,
+                        const int32_t *p0_dev, const int32_t *pos_rows, int rows_per_seq, int Hq, float scale,
+                        void *stream);
+/* bytes of the a16 buffer of T rows of n values (n % 32 == 0): T * n/32 * (16 + 1) half2 */
+size_t p1a_a16_bytes(int T, int n);
+/*
+ * Elementwise gate + a16 quantize over [T][n]: op 0: y = silu(a) * b, op 1: y = a * sigmoid(b); qbuf = a16(y).
+ * lda / ldb (0 = n) are the row strides of a and b; y is dense and may alias a when lda == n. n % 32 == 0.
+ * Replaces ew_quant (src/fast/fused.cuh:92-98, kernel src/fast/fused.cu:478-496).
+ */
+int p1a_ew_quant(int op, const float *a, const float *b, float *y, void *qbuf, int T, int n, int lda, int ldb, void *stream);
+
+/*
  * Chunked causal prefill: q, out [T][Hq][D] f32, query t at position p0 + t sees cache positions 0..p0+t of ONE
  * sequence (page table pt + (rtab ? rtab[0] : 0)); the cache must already hold positions 0..p0+T-1 (append first).
  * fp16 MFMA products with fp32 accumulation; gate as in p1a_attn_decode. `scratch` is caller-supplied device memory

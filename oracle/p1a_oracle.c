@@ -263,6 +263,52 @@ int orc_attn_prep(const float *qg, const float *k, const float *v, const float *
     return 0;
 }
 
+/*
+ * a16 activation quantize of the engine's quantized matvec (src/fast/matvec_a16.cu:29-100 quantize_a16, restated for
+ * fused producers in src/fast/a16q.cuh:21-45): per token row t of n values, per group g of 32 values
+ *   amax = max |v| (clamped to 65504 when it would round to an infinite f16), id = amax > 0 ? 1 / amax : 0,
+ *   w = v * id (rounded), sum = sum of w: the 4 values of a lane (lane l holds values 4l..4l+3) added in order from +0,
+ *   then the 8 lane sums in an xor butterfly with strides 4, 2, 1;
+ *   qbuf as half2 words: word (t * ng + g) * 16 + slot holds two scaled values, slot order of matvec_a16.cu:89-99;
+ *   word T * ng * 16 + t * ng + g holds (f16(amax), f16(sum)).
+ */
+void orc_a16_quant(const float *y, int T, int n, uint16_t *qbuf) {
+    const int ng = n / 32;
+    uint16_t *ads = qbuf + (size_t) T * ng * 16 * 2;
+    for (int t = 0; t < T; ++t)
+        for (int g = 0; g < ng; ++g) {
+            const float *v = y + (size_t) t * n + (size_t) g * 32;
+            float amax = 0.0f;
+            for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(v[i]));
+            amax = amax < 65520.0f ? amax : 65504.0f;
+            const float id = amax > 0.0f ? 1.0f / amax : 0.0f;
+            float w[32], ls[8];
+            for (int l = 0; l < 8; ++l) {
+                float sum = 0.0f;
+                for (int i = 0; i < 4; ++i) {
+                    w[4 * l + i] = v[4 * l + i] * id;
+                    sum = sum + w[4 * l + i];
+                }
+                ls[l] = sum;
+            }
+            for (int st = 4; st > 0; st >>= 1) {
+                float nx[8];
+                for (int l = 0; l < 8; ++l) nx[l] = ls[l] + ls[l ^ st];
+                memcpy(ls, nx, sizeof ls);
+            }
+            uint16_t *qs = qbuf + ((size_t) t * ng + g) * 16 * 2;
+            for (int l = 0; l < 8; ++l) {
+                const int off = l >= 4 ? 1 : 0, k = l - 4 * off;
+                qs[(4 * k + 0 + off) * 2 + 0] = orc_f32_to_f16(w[4 * l + 0]);
+                qs[(4 * k + 0 + off) * 2 + 1] = orc_f32_to_f16(w[4 * l + 2]);
+                qs[(4 * k + 2 + off) * 2 + 0] = orc_f32_to_f16(w[4 * l + 1]);
+                qs[(4 * k + 2 + off) * 2 + 1] = orc_f32_to_f16(w[4 * l + 3]);
+            }
+            ads[((size_t) t * ng + g) * 2 + 0] = orc_f32_to_f16(amax);
+            ads[((size_t) t * ng + g) * 2 + 1] = orc_f32_to_f16(ls[0]);
+        }
+}
+
 int orc_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

@@ -7,7 +7,7 @@ import os
 KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
-    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_decode", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
+    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_release", "p1a_last_error",
     "p1a_version",
 ]
@@ -49,6 +49,12 @@ def lib():
     L.p1a_kv_append.argtypes = [kvp, vp, vp, i32, vp, vp, i32, vp]
     L.p1a_attn_prep.restype = i32
     L.p1a_attn_prep.argtypes = [vp] * 8 + [kvp, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp]
+    L.p1a_attn_decode_a16.restype = i32
+    L.p1a_attn_decode_a16.argtypes = [vp, kvp, vp, vp, vp, i32, i32, vp, vp, i32, i32, f32, vp]
+    L.p1a_a16_bytes.restype = sz
+    L.p1a_a16_bytes.argtypes = [i32, i32]
+    L.p1a_ew_quant.restype = i32
+    L.p1a_ew_quant.argtypes = [i32, vp, vp, vp, vp, i32, i32, i32, i32, vp]
     L.p1a_attn_decode.restype = i32
     L.p1a_attn_decode.argtypes = [vp, kvp, vp, vp, i32, i32, vp, vp, i32, i32, f32, vp]
     L.p1a_attn_prefill.restype = i32
@@ -182,9 +188,19 @@ def attn_decode_dev(q, c, out, T, p0_dev, max_n, Hq, scale, gate=None):
     _check(lib().p1a_attn_decode(_ptr(q), ctypes.byref(c.struct()), _ptr(out), _ptr(gate), T, 0, _ptr(p0_dev), None, 0, Hq, scale, _stream()), "attn_decode_dev")
 
 
-def attn_decode_rows(q, c, out, T, pos, Hq, scale, gate=None, rows_per_seq=1):
-    """src/fast/attn.cuh:64-65; rows_per_seq > 1: consecutive rows form verify blocks that share one KV read."""
-    _check(lib().p1a_attn_decode(_ptr(q), ctypes.byref(c.struct()), _ptr(out), _ptr(gate), T, 0, None, _ptr(pos), rows_per_seq, Hq, scale, _stream()), "attn_decode_rows")
+def attn_decode_rows(q, c, out, T, pos, Hq, scale, gate=None, rows_per_seq=1, qbuf=None):
+    """src/fast/attn.cuh:64-65; rows_per_seq > 1: consecutive rows form verify blocks that share one KV read; qbuf: also
+    emit the a16 activation buffer of the gated rows (src/fast/fused.cu:478-496)."""
+    _check(lib().p1a_attn_decode_a16(_ptr(q), ctypes.byref(c.struct()), _ptr(out), _ptr(gate), _ptr(qbuf), T, 0, None, _ptr(pos), rows_per_seq, Hq, scale, _stream()), "attn_decode_rows")
+
+
+def a16_bytes(T, n):
+    return int(lib().p1a_a16_bytes(T, n))
+
+
+def ew_quant(op, a, b, y, qbuf, T, n, lda=0, ldb=0):
+    """src/fast/fused.cuh:92-98: op 0 y = silu(a) * b, op 1 y = a * sigmoid(b); qbuf = a16(y)."""
+    _check(lib().p1a_ew_quant(op, _ptr(a), _ptr(b), _ptr(y), _ptr(qbuf), T, n, lda, ldb, _stream()), "ew_quant")
 
 
 def prefill_scratch_bytes(T, p0, Hq, Hkv, D):

@@ -129,10 +129,32 @@ int p1a_attn_prep(const float * qg, const float * k, const float * v, const floa
     return launch_prep(*c, qg, k, v, q_norm, k_norm, pos, q, gate, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, (hipStream_t) stream);
 }
 
+size_t p1a_a16_bytes(int T, int n) { return T < 0 || n < 0 ? 0 : (size_t) T * (size_t) (n / 32) * 17 * 4; }
+
+int p1a_ew_quant(int op, const float * a, const float * b, float * y, void * qbuf, int T, int n, int lda, int ldb, void * stream) {
+    if (!a || !b || !y || !qbuf || T < 0 || (op != 0 && op != 1)) { set_error("p1a_ew_quant: null argument, negative T or unknown op"); return P1A_E_ARG; }
+    if (T == 0) return P1A_OK;
+    if (!lda) lda = n;
+    if (!ldb) ldb = n;
+    const uintptr_t al = (uintptr_t) a | (uintptr_t) b | (uintptr_t) y | (uintptr_t) qbuf;
+    if (n < 32 || n % 32 || (al & 15) || ((lda | ldb) & 3) || lda < n || ldb < n || T > 65535 || (y == a && lda != n)) {
+        set_error("p1a_ew_quant: n %% 32 == 0, 16-byte aligned pointers, row strides multiples of 4 and >= n (y may alias a only when dense)");
+        return P1A_E_SHAPE;
+    }
+    return launch_ew_quant(op, a, b, y, qbuf, T, n, lda, ldb, (hipStream_t) stream);
+}
+
 int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float * gate, int T, int p0,
                     const int32_t * p0_dev, const int32_t * pos_rows, int rows_per_seq, int Hq, float scale,
                     void * stream) {
+    return p1a_attn_decode_a16(q, c, out, gate, nullptr, T, p0, p0_dev, pos_rows, rows_per_seq, Hq, scale, stream);
+}
+
+int p1a_attn_decode_a16(const float * q, const p1a_kv * c, float * out, const float * gate, void * qbuf, int T, int p0,
+                        const int32_t * p0_dev, const int32_t * pos_rows, int rows_per_seq, int Hq, float scale,
+                        void * stream) {
     if (!kv_ok(c, "p1a_attn_decode")) return P1A_E_ARG;
+    if (qbuf && (((uintptr_t) qbuf & 15) || (Hq * c->D) % 32)) { set_error("p1a_attn_decode: qbuf must be 16-byte aligned and Hq*D %% 32 == 0"); return P1A_E_SHAPE; }
     if (!q || !out) { set_error("p1a_attn_decode: null q/out"); return P1A_E_ARG; }
     if (T < 1 || T > P1A_MAX_ROWS || Hq < c->Hkv || Hq % c->Hkv) {
         set_error("p1a_attn_decode: unsupported shape (D=%d Hq=%d Hkv=%d T=%d)", c->D, Hq, c->Hkv, T);
@@ -150,6 +172,7 @@ int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float 
     a.nsplit = nsplit_req();
     a.cus = cu_count();
     a.skip_merge = g_skip_merge;
+    a.qbuf = qbuf;
     size_t need_o, need_ml;
     decode_scratch_need(*c, Hq, T < 8 ? 8 : T, a.rows_per_group, a.nsplit, a.cus, need_o, need_ml);
     scratch * sc = scratch_for(s, need_o, need_ml);

@@ -219,6 +219,32 @@ int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, co
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
+namespace {
+// elementwise gate + a16 quantize, one float4 per lane, 8 lanes per 32-value group (src/fast/fused.cu:478-496):
+// OP 0: y = silu(a) * b (the MLP gate); OP 1: y = a * sigmoid(b) (the attention output gate). y may alias a.
+template <int OP>
+__global__ void __launch_bounds__(256) ew_q_k(const float * a, const float * b, float * y, void * qbuf, int n, int lda, int ldb) {
+    const int n4 = n >> 2, t = blockIdx.y, T = gridDim.y;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const bool act = i < n4;
+    f4 o = {0.f, 0.f, 0.f, 0.f};
+    if (act) {
+        const f4 av = reinterpret_cast<const f4 *>(a + (size_t) t * lda)[i], bv = reinterpret_cast<const f4 *>(b + (size_t) t * ldb)[i];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = OP == 0 ? (av[e] / (1.0f + expf(-av[e]))) * bv[e] : av[e] * (1.0f / (1.0f + expf(-bv[e])));
+        reinterpret_cast<f4 *>(y + (size_t) t * n)[i] = o;
+    }
+    a16_quant8(o, i & 7, qbuf, t, i >> 3, n >> 5, T, act);   // n % 32 == 0: dead lanes form whole groups
+}
+}   // namespace
+
+int launch_ew_quant(int op, const float * a, const float * b, float * y, void * qbuf, int T, int n, int lda, int ldb, hipStream_t s) {
+    const dim3 grid((n / 4 + 255) / 256, T);
+    if (op == 0) ew_q_k<0><<<grid, 256, 0, s>>>(a, b, y, qbuf, n, lda, ldb);
+    else ew_q_k<1><<<grid, 256, 0, s>>>(a, b, y, qbuf, n, lda, ldb);
+    return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
+}
+
 int launch_prep(const p1a_kv & c, const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
                 const int32_t * pos, float * q, float * gate, int p0, int T, int Hq, int n_rot, float freq_base, float eps,
                 int ldq, int ldk, int ldv, hipStream_t s) {

@@ -44,6 +44,37 @@ constexpr size_t head_bytes(uint32_t type, int D) {
     return type == P1A_KV_F16 ? (size_t) D * 2 : type == P1A_KV_Q8_0 ? (size_t) (D / 32) * 34 : (size_t) (D / 32) * 18;
 }
 
+// ---- a16 activation quantize of one 32-value group (src/fast/a16q.cuh:21-45 of the reference) ----
+// Lane l8 (0..7) of an aligned 8-lane segment holds values 4 l8 .. 4 l8 + 3 of the group; all 8 lanes call together.
+// qbuf layout: half2 words; word (t * ng + g) * 16 + slot = two scaled values (slot order of the engine), word
+// T * ng * 16 + t * ng + g = (amax, sum of the scaled values). Products and sums are rounded one by one (no contraction),
+// the sum runs over a lane's 4 values in order from +0 and then over the lanes in an xor butterfly with strides 4, 2, 1.
+#if defined(__HIPCC__)
+__device__ __forceinline__ void a16_quant8(const f4 v4, int l8, void * qbuf, int t, int g, int ng, int T, bool store) {
+#pragma clang fp contract(off)
+    float v[4] = {v4[0], v4[1], v4[2], v4[3]};
+    float amax = fmaxf(0.0f, fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3]))));
+#pragma unroll
+    for (int st = 4; st > 0; st >>= 1) amax = fmaxf(amax, __shfl_xor(amax, st));
+    amax = amax < 65520.0f ? amax : 65504.0f;               // a finite f16 scale
+    const float id = amax > 0.0f ? 1.0f / amax : 0.0f;
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[i] = v[i] * id;
+        sum = sum + v[i];
+    }
+#pragma unroll
+    for (int st = 4; st > 0; st >>= 1) sum = sum + __shfl_xor(sum, st);
+    if (!store) return;
+    h2 * qs = reinterpret_cast<h2 *>(qbuf) + ((size_t) t * ng + g) * 16;
+    if (l8 == 0) reinterpret_cast<h2 *>(qbuf)[(size_t) T * ng * 16 + (size_t) t * ng + g] = h2{(half_t) amax, (half_t) sum};
+    const int off = l8 >= 4 ? 1 : 0, k = l8 - 4 * off;
+    qs[4 * k + 0 + off] = h2{(half_t) v[0], (half_t) v[2]};
+    qs[4 * k + 2 + off] = h2{(half_t) v[1], (half_t) v[3]};
+}
+#endif
+
 // host-side launch entry points implemented in the .hip files
 int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, const int32_t * p0_dev,
                   const int32_t * pos_rows, int T, hipStream_t s);
@@ -63,6 +94,7 @@ struct decode_args {
     bool skip_merge;      // benchmarks only: stop after the split-K kernel
     float * part_o;       // [T*Hq][nsplit][D]
     float * part_ml;      // [T*Hq][nsplit][2]
+    void * qbuf;          // optional: a16 activation buffer of the (gated) output, [T][Hq*D] values
 };
 int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s);
 int decode_rows_per_group(const p1a_kv & c, int Hq, int want);
@@ -72,6 +104,7 @@ void decode_scratch_need(const p1a_kv & c, int Hq, int rows, int rows_per_group,
 int launch_prep(const p1a_kv & c, const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
                 const int32_t * pos, float * q, float * gate, int p0, int T, int Hq, int n_rot, float freq_base, float eps,
                 int ldq, int ldk, int ldv, hipStream_t s);
+int launch_ew_quant(int op, const float * a, const float * b, float * y, void * qbuf, int T, int n, int lda, int ldb, hipStream_t s);
 int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s);
 int launch_sigmoid_mul(float * x, const float * g, size_t n, hipStream_t s);

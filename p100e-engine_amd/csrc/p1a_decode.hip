@@ -625,7 +625,8 @@ __global__ void __launch_bounds__(256) dec_generic_k(const gen_params P) {
 // One wave per (row, 32 dims): lane = (slice of the splits, 4 dims); slice k folds splits k, k + 8, ... in order and
 // the 8 slices are then added in order, so the result depends on nothing but the partials.
 __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o, const float * __restrict__ part_ml,
-                                              float * __restrict__ out, const float * __restrict__ gate, int NS, int D) {
+                                              float * __restrict__ out, const float * __restrict__ gate, int NS, int D,
+                                              void * qbuf, int Hq, int T) {
     __shared__ f4 sacc[8][8];
     __shared__ float sden[8];
     const size_t row = blockIdx.x;
@@ -689,6 +690,12 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
             for (int x = 0; x < 4; ++x) r[x] *= 1.0f / (1.0f + expf(-gt[x]));
         }
         *reinterpret_cast<f4 *>(out + row * D + d) = r;
+        // the 8 lanes of slice 0 hold one 32-value group of the output row: its a16 activation quantize rides along
+        // (what the engine's ew_quant emits for the output projection, src/fast/fused.cu:478-496)
+        if (qbuf) {
+            const int t = (int) (row / Hq), h = (int) (row - (size_t) t * Hq);
+            a16_quant8(r, q4, qbuf, t, h * (D >> 5) + (int) blockIdx.y, (Hq * D) >> 5, T, true);
+        }
     }
 }
 
@@ -821,7 +828,7 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
         rc = hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
     }
     if (rc != P1A_OK || a.skip_merge) return rc;
-    merge_k<<<dim3(a.T * a.Hq, c.D / 32), 64, 0, s>>>(a.part_o, a.part_ml, a.out, a.gate, pl.NS, c.D);
+    merge_k<<<dim3(a.T * a.Hq, c.D / 32), 64, 0, s>>>(a.part_o, a.part_ml, a.out, a.gate, pl.NS, c.D, a.qbuf, a.Hq, a.T);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 

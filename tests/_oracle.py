@@ -46,6 +46,7 @@ def lib():
         L.orc_rmsnorm_heads.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_float]
         L.orc_attn_prep.argtypes = [ctypes.c_void_p] * 8 + [ctypes.POINTER(orc_kv)] + [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 3
         L.orc_attn_prep.restype = ctypes.c_int
+        L.orc_a16_quant.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         L.orc_num_threads.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -163,3 +164,13 @@ def attn_prep(c, qg, k, v, q_norm, k_norm, pos, p0, Hq, n_rot, freq_base, eps=1e
                              c.Hkv, c.D, n_rot, freq_base, eps, 0, 0, 0)
     assert rc == 0, rc
     return q, gate
+
+
+def a16_quant(y):
+    """y [T][n] f32 -> the engine's a16 activation buffer as uint16 halves: [T*ng*16*2] values then [T*ng*2] (amax, sum)"""
+    y = np.ascontiguousarray(y, np.float32)
+    T, n = y.shape
+    ng = n // 32
+    q = np.zeros(T * ng * 34, np.uint16)
+    lib().orc_a16_quant(_p(y), T, n, _p(q))
+    return q

@@ -110,3 +110,59 @@ def test_refusals(p1a):
     with pytest.raises(p1a.P1AError):       # row stride shorter than a row
         p1a.attn_prep(z, z, z, None, None, pos, z, z, c, 0, 1, 4, 64, 1e7, 1e-6, ldq=64)
     torch.cuda.synchronize()
+
+
+def test_ew_quant_sigmoid_and_silu(p1a):
+    """gate + a16 emit (src/fast/fused.cu:478-496): y within fp32 rounding of the oracle, the a16 bytes exactly the oracle's
+    quantization of the y the GPU wrote; strided a / b; y aliasing a"""
+    T, n = 3, 6144
+    g = I.rng(41)
+    a = I.normal(g, (T, n)) * 2.0
+    b = I.normal(g, (T, n))
+    a[1, 64:96] = 0.0                                           # an all-zero group
+    lda, ldb = n + 8, n + 32
+    ap = np.zeros((T, lda), np.float32); ap[:, :n] = a
+    bp = np.zeros((T, ldb), np.float32); bp[:, :n] = b
+    for op in (1, 0):
+        y = torch.zeros((T, n), device="cuda")
+        qb = torch.zeros(p1a.a16_bytes(T, n) // 2, dtype=torch.int16, device="cuda")
+        p1a.ew_quant(op, dev(ap), dev(bp), y, qb, T, n, lda=lda, ldb=ldb)
+        torch.cuda.synchronize()
+        yh = y.cpu().numpy()
+        if op == 1:
+            ref = a.astype(np.float64) / (1.0 + np.exp(-b.astype(np.float64)))
+        else:
+            ref = a.astype(np.float64) / (1.0 + np.exp(-a.astype(np.float64))) * b.astype(np.float64)
+        assert np.max(np.abs(yh - ref)) <= 4e-7 * max(1.0, np.abs(ref).max())
+        assert np.array_equal(qb.cpu().numpy().view(np.uint16), O.a16_quant(yh)), op
+    # in place: y aliases a (dense rows)
+    ya = dev(a)
+    qb = torch.zeros(p1a.a16_bytes(T, n) // 2, dtype=torch.int16, device="cuda")
+    p1a.ew_quant(1, ya, dev(b), ya, qb, T, n)
+    torch.cuda.synchronize()
+    assert np.array_equal(qb.cpu().numpy().view(np.uint16), O.a16_quant(ya.cpu().numpy()))
+    with pytest.raises(p1a.P1AError):
+        p1a.ew_quant(1, ya, dev(b), ya, qb, T, n - 4)          # n % 32 != 0
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("kv_type", [O.KV_Q8_0, O.KV_F16])
+def test_decode_emits_a16(p1a, kv_type):
+    """the decode call with a qbuf: same output bits as without, and qbuf = a16(gated output)"""
+    from _gpu import Pool
+    Hq, Hkv, D, psh = 24, 4, 256, 6
+    lens = [300, 77]
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=13)
+    T = 3
+    q, _, _, gate = I.qkv(61, 1, T, Hq, Hkv, D)
+    pos = np.array([299, 76, 150], np.int32)
+    rt = np.array([0, pool.maxp, 0], np.int32)
+    c = pool.devkv.with_rows(dev(rt))
+    o1 = torch.zeros((T, Hq, D), device="cuda"); o2 = torch.zeros((T, Hq, D), device="cuda")
+    qb = torch.zeros(p1a.a16_bytes(T, Hq * D) // 2, dtype=torch.int16, device="cuda")
+    dq, dg, dp = dev(q), dev(gate), dev(pos)
+    p1a.attn_decode_rows(dq, c, o1, T, dp, Hq, 1 / 16, gate=dg)
+    p1a.attn_decode_rows(dq, c, o2, T, dp, Hq, 1 / 16, gate=dg, qbuf=qb)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2)
+    assert np.array_equal(qb.cpu().numpy().view(np.uint16), O.a16_quant(o2.cpu().numpy().reshape(T, Hq * D)))

@@ -111,3 +111,54 @@ def test_kv_rows_are_the_append_of_the_roped_k(kv_type):
     O.attn_prep(c3, qg, k, v, qn, kn, pos, 3, Hq, n_rot, base)
     O.kv_append_rows(c4, kr, v, 3 + np.arange(T))
     assert np.array_equal(c3.k, c4.k) and np.array_equal(c3.v, c4.v)
+
+
+def np_a16(y):
+    """independent float32 restatement of the a16 activation quantize (src/fast/matvec_a16.cu:29-100): the slot of each
+    element is written out from the engine's comment 'lanes holding elements 0..15 write outputs 4k+0 / 4k+2; those
+    holding 16..31 write 4k+1 / 4k+3', lane = 4 consecutive elements, pairs (v0, v2) and (v1, v3)"""
+    T, n = y.shape
+    ng = n // 32
+    out = np.zeros((T, ng, 16, 2), np.float16)
+    ads = np.zeros((T, ng, 2), np.float16)
+    for t in range(T):
+        for g in range(ng):
+            v = y[t, 32 * g:32 * g + 32].astype(np.float32)
+            amax = np.float32(np.abs(v).max())
+            if not amax < np.float32(65520.0):
+                amax = np.float32(65504.0)
+            idv = np.float32(1.0) / amax if amax > 0 else np.float32(0.0)
+            w = (v * idv).astype(np.float32)
+            for x in range(32):
+                hi, xx = x // 16, x % 16
+                k, i = xx // 4, xx % 4
+                out[t, g, 4 * k + 2 * (i & 1) + hi, i >> 1] = np.float16(w[x])
+            lane = [np.float32(0.0)] * 8
+            for l in range(8):
+                s_ = np.float32(0.0)
+                for i in range(4):
+                    s_ = np.float32(s_ + w[4 * l + i])
+                lane[l] = s_
+            for st in (4, 2, 1):
+                lane = [np.float32(lane[l] + lane[l ^ st]) for l in range(8)]
+            ads[t, g] = (np.float16(amax), np.float16(lane[0]))
+    return np.concatenate([out.reshape(-1).view(np.uint16), ads.reshape(-1).view(np.uint16)])
+
+
+def test_a16_quant_against_numpy_and_closed_forms():
+    g = I.rng(31)
+    y = (I.normal(g, (3, 256)) * np.array([[1.0], [300.0], [1e-3]], np.float32)).astype(np.float32)
+    y[0, 32:64] = 0.0                     # an all-zero group: amax 0, scale 0, every value 0
+    y[1, 64:96] = 1.0                     # a unit group: every value 1, sum 32
+    y[2, 0] = 7.0e4                       # above the f16 range: the stored scale clamps to 65504, values scale by 1 / 65504
+    got = O.a16_quant(y)
+    assert np.array_equal(got, np_a16(y))
+    ng = 8
+    vals = got[: 3 * ng * 32].view(np.float16).reshape(3, ng, 32)
+    ads = got[3 * ng * 32:].view(np.float16).reshape(3, ng, 2)
+    assert np.all(vals[0, 1] == 0) and ads[0, 1, 0] == 0 and ads[0, 1, 1] == 0
+    assert np.all(vals[1, 2] == 1) and ads[1, 2, 0] == 1 and ads[1, 2, 1] == 32
+    assert ads[2, 0, 0] == np.float16(65504.0) and np.isfinite(vals[2, 0].astype(np.float32)).all()
+    assert np.float32(vals[2, 0].astype(np.float32).max()) > 1.0      # |v| / 65504 passes 1 for the clamped group
+    # every scaled value is v / amax: the largest magnitude of an ordinary group is exactly 1
+    assert np.abs(vals[0, 0].astype(np.float32)).max() == 1.0
