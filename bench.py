@@ -106,11 +106,17 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
     out = torch.empty((T, Hq, D), device="cuda")
     kc = normed((T, Hkv, D))
     vc = torch.randn((T, Hkv, D), generator=g, device="cuda")
-    sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=5)
+    # the caller-scratch variant (what attn_fold callers get): the cache is converted to f16 once per call
+    scr = torch.empty(p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D), dtype=torch.uint8, device="cuda")
+    sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate, scratch=scr), reps=5)
     flop = 4.0 * D * Hq * (p0 * T + T * (T + 1) / 2)
     ex["prefill_T4096_p28672_q8_0_ms"] = round(sec * 1e3, 4)
     ex["prefill_TFLOPs"] = round(flop / sec / 1e12, 1)
     ex["prefill_frac_of_f16_mfma_peak"] = round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)
+    ex["prefill_scratch_MB"] = round(scr.numel() / 1e6, 1)
+    sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=5)
+    ex["prefill_no_scratch_ms"] = round(sec * 1e3, 4)
+    del scr
     sec = time_eager(torch, lambda: p1a.kv_append(c, kc, vc, p0, T), reps=20)
     ab = 2 * T * Hkv * D * 4 + 2 * T * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
     ex["append_T4096_q8_0_us"] = round(sec * 1e6, 2)
@@ -213,7 +219,8 @@ def main():
         qp = torch.randn((T, Hq, D), device="cuda").half().float()
         gp = torch.randn((T, Hq * D), device="cuda")
         op = torch.empty((T, Hq, D), device="cuda")
-        sec = time_eager(torch, lambda: p1a.attn_prefill(qp, c, op, T, p0, Hq, scale, gate=gp), reps=3, warmup=1)
+        scr = torch.empty(p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D), dtype=torch.uint8, device="cuda")
+        sec = time_eager(torch, lambda: p1a.attn_prefill(qp, c, op, T, p0, Hq, scale, gate=gp, scratch=scr), reps=3, warmup=1)
         flop = 4.0 * D * Hq * (p0 * T + T * (T + 1) / 2)
         print(json.dumps({"prefill_T4096_p28672_q8_0_ms": round(sec * 1e3, 4), "TFLOPs": round(flop / sec / 1e12, 1)}))
         return

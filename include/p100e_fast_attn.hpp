@@ -138,9 +138,12 @@ inline bool attn_prefill_variant(const float * q, const kv_cache & c, float * ou
                                  hipStream_t s, int /*variant: one kernel here*/) {
     return attn_prefill(q, c, out, T, p0, Hq, scale, s);
 }
-// src/fast/attn_fold.cuh:19-26 (chunk / nsplit are accepted and ignored: the kernel keeps P and the dequantized tiles on chip)
-inline size_t attn_fold_scratch_bytes(int T, int Hkv, int /*chunk*/, int /*nsplit*/) {
-    return p1a_attn_prefill_scratch_bytes(T, 0, 6 * Hkv, Hkv, 256);
+// src/fast/attn_fold.cuh:19-26 (chunk / nsplit are accepted and ignored: P never leaves the chip). The scratch is optional
+// here: a buffer of attn_fold_scratch_bytes(T, Hkv, ..., p0) bytes lets a quantized cache be converted to f16 once per
+// call; the reference's own size (which knows nothing of p0) is accepted too and simply selects the on-the-fly kernel
+// when it is too small.
+inline size_t attn_fold_scratch_bytes(int T, int Hkv, int /*chunk*/, int /*nsplit*/, int p0 = 0) {
+    return p1a_attn_prefill_scratch_bytes(T, p0, 6 * Hkv, Hkv, 256);
 }
 inline bool attn_fold(const float * q, const kv_cache & c, float * out, int T, int p0, int Hq, float scale, void * scratch,
                       size_t scratch_bytes, hipStream_t s, int /*chunk*/ = 0, int /*nsplit*/ = 0, const float * gate = nullptr) {

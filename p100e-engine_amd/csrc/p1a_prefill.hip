@@ -20,6 +20,7 @@
 #include "p1a_common.hpp"
 
 namespace p1a {
+size_t prefill_stage_bytes(int n, int Hkv, int D);
 namespace {
 
 constexpr int BM = 128;   // query tokens per workgroup
@@ -597,9 +598,60 @@ int launch_pf(const pf_params & P, hipStream_t s) {
 
 }   // namespace
 
+namespace {
+// Staging pass of the scratch variant: positions 0 .. n-1 of one sequence of a q8_0 / q4_0 cache -> contiguous f16 rows
+// [n][Hkv][D] (K, then V). Same conversion as the in-kernel stagers (code * f16 scale, rounded once to f16), so the
+// attention kernel sees the very tiles it would have built itself. One thread per 16 codes (q8_0) / per block (q4_0).
+template <uint32_t KT>
+__global__ void __launch_bounds__(256) dq_k(const char * kc, const char * vc, kv_view pg, int n, int Hkv, int D, char * ko, char * vo) {
+    const int32_t * ptab = pg.pt ? (pg.rtab ? pg.pt + pg.rtab[0] : pg.pt) : nullptr;
+    const int per = KT == P1A_KV_Q8_0 ? 16 : 32;               // values per item
+    const int ipr = Hkv * D / per;                             // items per position
+    const long long idx = (long long) blockIdx.x * 256 + threadIdx.x;
+    const int row = (int) (idx / ipr), it = (int) (idx - (long long) row * ipr);
+    if (row >= n) return;
+    const size_t off = kv_off_tab(pg, ptab, row);
+    const int iph = D / per, h = it / iph, cc = it - h * iph;
+    const size_t orow = ((size_t) row * Hkv + h) * D * 2;
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const char * src = (which ? vc : kc) + off;
+        char * dst = (which ? vo : ko) + orow;
+        if constexpr (KT == P1A_KV_Q8_0) {
+            const char * head = src + (size_t) h * (D / 32) * 34;
+            const u4 w = *reinterpret_cast<const u4 *>(head + (D / 32) * 2 + cc * 16);
+            const uint32_t d16 = *reinterpret_cast<const uint16_t *>(head + (cc >> 1) * 2);
+            const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
+            const pair32 x0 = deq8x4(w[0], dd), x1 = deq8x4(w[1], dd), x2 = deq8x4(w[2], dd), x3 = deq8x4(w[3], dd);
+            u4 * o = reinterpret_cast<u4 *>(dst + cc * 32);
+            o[0] = u4{x0.lo, x0.hi, x1.lo, x1.hi};
+            o[1] = u4{x2.lo, x2.hi, x3.lo, x3.hi};
+        } else {
+            const uint16_t * blk = reinterpret_cast<const uint16_t *>(src + ((size_t) h * (D / 32) + cc) * 18);
+            const uint32_t d16 = blk[0];
+            const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
+            pair32 lo[4], hi[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t w = (uint32_t) blk[1 + 2 * k] | ((uint32_t) blk[2 + 2 * k] << 16);
+                lo[k] = deq4x4(w & 0x0f0f0f0fu, dd);
+                hi[k] = deq4x4((w >> 4) & 0x0f0f0f0fu, dd);
+            }
+            u4 * o = reinterpret_cast<u4 *>(dst + cc * 64);
+            o[0] = u4{lo[0].lo, lo[0].hi, lo[1].lo, lo[1].hi};
+            o[1] = u4{lo[2].lo, lo[2].hi, lo[3].lo, lo[3].hi};
+            o[2] = u4{hi[0].lo, hi[0].hi, hi[1].lo, hi[1].hi};
+            o[3] = u4{hi[2].lo, hi[2].hi, hi[3].lo, hi[3].hi};
+        }
+    }
+}
+}   // namespace
+
+// bytes of the f16 staging copy of the first n positions (K and V)
+size_t prefill_stage_bytes(int n, int Hkv, int D) { return 2 * (size_t) n * Hkv * D * 2; }
+
 int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s) {
-    (void) scratch; (void) scratch_bytes;
     if (c.D != 64 && c.D != 128 && c.D != 256) { set_error("p1a_attn_prefill: unsupported head size D=%d", c.D); return P1A_E_SHAPE; }
     if ((((uintptr_t) c.k | (uintptr_t) c.v) & 15) || (c.pt && (c.pstride & 15))) { set_error("p1a_attn_prefill: cache base / page stride must be 16-byte aligned"); return P1A_E_SHAPE; }
     pf_params P;
@@ -609,6 +661,23 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
     P.nblk = (T + BM - 1) / BM;
 #define PF(KT_) (c.D == 256 ? launch_pf<KT_, 256>(P, s) : c.D == 128 ? launch_pf<KT_, 128>(P, s) : launch_pf<KT_, 64>(P, s))
     if (c.type == P1A_KV_F16) return PF(P1A_KV_F16);
+    // A quantized cache with enough caller scratch: convert the visible positions to f16 once (tens of microseconds, the
+    // copy stays in the Infinity Cache) and run the f16 kernel on it - every workgroup then skips the dequantization it
+    // would otherwise repeat per 128 query rows. Same tiles, same products, same bits as the direct kernel.
+    const int n = p0 + T;
+    static const bool no_stage = getenv("P1A_PF_NOSTAGE") && atoi(getenv("P1A_PF_NOSTAGE"));   // development A/B switch
+    if (!no_stage && scratch && !((uintptr_t) scratch & 255) && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D)) {
+        char * ko = (char *) scratch, * vo = ko + (size_t) n * c.Hkv * c.D * 2;
+        const long long items = (long long) n * (c.Hkv * c.D / (c.type == P1A_KV_Q8_0 ? 16 : 32));
+        const unsigned blocks = (unsigned) ((items + 255) / 256);
+        if (c.type == P1A_KV_Q8_0) dq_k<P1A_KV_Q8_0><<<blocks, 256, 0, s>>>(P.kc, P.vc, P.pg, n, c.Hkv, c.D, ko, vo);
+        else dq_k<P1A_KV_Q4_0><<<blocks, 256, 0, s>>>(P.kc, P.vc, P.pg, n, c.Hkv, c.D, ko, vo);
+        if (hipPeekAtLastError() != hipSuccess) return P1A_E_LAUNCH;
+        P.kc = ko; P.vc = vo;
+        P.pg.pt = nullptr; P.pg.rtab = nullptr; P.pg.psh = 0; P.pg.pstride = 0;
+        P.pg.rowb = (size_t) c.Hkv * c.D * 2;
+        return PF(P1A_KV_F16);
+    }
     if (c.type == P1A_KV_Q8_0) return PF(P1A_KV_Q8_0);
     return PF(P1A_KV_Q4_0);
 #undef PF
@@ -621,6 +690,9 @@ extern "C" void p1a_set_pf_trace(long long * buf) { (void) hipMemcpyToSymbol(HIP
 #endif
 
 extern "C" size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D) {
-    (void) T; (void) p0; (void) Hq; (void) Hkv; (void) D;
-    return 0;   // the kernel keeps every intermediate in registers and LDS
+    (void) Hq;
+    if (T < 1 || p0 < 0 || Hkv < 1 || D < 1) return 0;
+    // optional: with this much scratch a quantized cache is converted to f16 once per call instead of once per
+    // workgroup; with less (or none) the kernel converts on the fly and needs nothing
+    return p1a::prefill_stage_bytes(p0 + T, Hkv, D);
 }

@@ -81,3 +81,23 @@ def test_prefill_rows_match_decode(p1a, kv_type):
     torch.cuda.synchronize()
     ma, rl = I.errors(out, dec.cpu().numpy())
     assert ma < 1e-3 and rl < 5e-4, (ma, rl)
+
+
+@pytest.mark.parametrize("kv_type", [O.KV_Q8_0, O.KV_Q4_0])
+@pytest.mark.parametrize("Hq,Hkv,D,psh", [(12, 2, 256, 5), (8, 2, 128, 4)])
+def test_scratch_variant_gives_the_same_bits(p1a, kv_type, Hq, Hkv, D, psh):
+    """with caller scratch the quantized cache is converted to f16 once and the f16 kernel runs on the copy: same tiles,
+    same products, same bits as the on-the-fly kernel; a scratch that is too small silently takes the direct kernel"""
+    p0, T = 777, 300
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [p0 + T, 40], seed=3 + psh, n_layers=2, layer=0)
+    q, _, _, gate = I.qkv(70 + D, 1, T, Hq, Hkv, D, f16_inputs=True)
+    a = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16, gate=gate)
+    need = p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D)
+    assert need == 2 * (p0 + T) * Hkv * D * 2
+    dq, dg = dev(q), dev(gate)
+    for nbytes in (need, need // 2):
+        scr = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        out = torch.zeros((T, Hq, D), device="cuda")
+        p1a.attn_prefill(dq, pool.dev_seq(0), out, T, p0, Hq, 1 / 16, gate=dg, scratch=scr)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), a), nbytes
