@@ -29,12 +29,33 @@ constexpr int NTHR = 256;
 constexpr float NEG_INF = -__builtin_inff();
 
 template <int D> struct pf_cfg {
-    static constexpr int KSTR = D * 2 + 16;    // K tile row stride (odd multiple of 16 B: conflict-free b128 reads)
-    static constexpr int VSTR = D * 2 + 32;    // V tile row stride (4 consecutive rows cover disjoint banks for tr16)
-    static constexpr int KT_B = BN * KSTR, VT_B = BN * VSTR;
-    static constexpr int STAGE_B = KT_B + VT_B;
     static constexpr int NKS = D / 16;         // k-steps of S^T (16 dims each)
     static constexpr int NDT = D / 32;         // 32-dim tiles of O^T
+};
+
+// Where the f16 tiles sit in LDS: in blocks of two rows (2 x 2 D bytes, then padding). Block (key & 7) + 8 (key >> 4)
+// holds key in its half (key >> 3) & 1 - two keys of the same 16-key group. For D = 256 a block is exactly what one
+// global_load_lds_dwordx4 moves (64 lanes x 16 bytes to 1 KB of consecutive LDS), and one page base serves it; tiles
+// staged through registers use the same places. The padding puts the rows that are read together into disjoint banks:
+// S^T row c of half u is the key of block 16 u + (c & 15), half c >> 4 (16 consecutive lanes: 16 blocks, 4 banks
+// apart); the transposing V reads take 4 consecutive blocks of one half (16 banks apart). Every read address is
+// (per-lane base) + (compile-time offset).
+template <int D> struct pf_lay {
+    static constexpr int RB = 2 * D;                            // bytes of a row
+    static constexpr int KB = 2 * RB + 16, VB = 2 * RB + 64;   // block strides
+    static constexpr int KT_B = 32 * KB, VT_B = 32 * VB;
+    static constexpr int STAGE_B = KT_B + VT_B;
+    static __device__ __forceinline__ int key_off(int key, int bstride) { return ((key & 7) + 8 * (key >> 4)) * bstride + ((key >> 3) & 1) * RB; }
+    // S^T operand rows: lane base of row c, offset of half u
+    static __device__ __forceinline__ int k_lane(int c) { return (c & 15) * KB + (c >> 4) * RB; }
+    static constexpr int k_half(int u) { return 16 * u * KB; }
+    // which key of the tile value i of half u of a lane's S^T column is, without the lane's 4 g
+    static constexpr int key_of(int u, int i) { return 32 * u + 16 * ((i >> 2) & 1) + 8 * (i >> 3) + (i & 3); }
+    // V^T operand of k-step ps: rows r = 4 g + kk (lane part), then the step's two row groups:
+    // keys 32 (ps / 2) + 8 (ps % 2) + r and the same + 16
+    static __device__ __forceinline__ int v_lane(int r) { return r * VB; }
+    static constexpr int v_lo(int ps) { return 16 * (ps >> 1) * VB + (ps & 1) * RB; }
+    static constexpr int v_hi(int ps) { return v_lo(ps) + 8 * VB; }
 };
 
 #ifdef P1A_TRACE
@@ -84,6 +105,7 @@ constexpr float RESCALE_STEP = 8.0f;   // log2 units: the reference maximum of a
 // of the wave size, so it sits in scalar registers), vo = the loop-invariant 32-bit offset of the item inside its group
 // (row in the group * row bytes + offs()[n]); the loads then need no address arithmetic at all.
 typedef unsigned u2v __attribute__((ext_vector_type(2)));
+typedef float f2v __attribute__((ext_vector_type(2)));
 typedef uint32_t __attribute__((may_alias)) u32a;   // the parked scale blocks are written as dwords and read as halves
 typedef uint16_t __attribute__((may_alias)) u16a;
 typedef const __attribute__((address_space(1))) char * gptr;      // global memory, so the loads are global_load (vmcnt only)
@@ -120,7 +142,7 @@ template <int D> struct stager<P1A_KV_Q8_0, D> {
         const uint32_t d16 = r.d[x];
         const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
         const pair32 x0 = deq8x4(r.w[x][2 * part], dd), x1 = deq8x4(r.w[x][2 * part + 1], dd);
-        *reinterpret_cast<u4 *>(tile + key * stride + cc * 32 + part * 16) = u4{x0.lo, x0.hi, x1.lo, x1.hi};
+        *reinterpret_cast<u4 *>(tile + pf_lay<D>::key_off(key, stride) + cc * 32 + part * 16) = u4{x0.lo, x0.hi, x1.lo, x1.hi};
     }
 };
 
@@ -139,7 +161,7 @@ template <int D> struct stager<P1A_KV_F16, D> {
     static constexpr int PARTS = 1;
     static __device__ __forceinline__ void store_part(const raw & r, char * tile, int stride, int tid, int x, int) {
         const int key = item_map<CPK>::key(x, tid), cc = item_map<CPK>::cc(x, tid);
-        *reinterpret_cast<u4 *>(tile + key * stride + cc * 16) = r.w[x];
+        *reinterpret_cast<u4 *>(tile + pf_lay<D>::key_off(key, stride) + cc * 16) = r.w[x];
     }
 };
 
@@ -173,7 +195,7 @@ template <int D> struct stager<P1A_KV_Q4_0, D> {
             const uint32_t w = (uint32_t) r.h[x][1 + 2 * kb] | ((uint32_t) r.h[x][2 + 2 * kb] << 16);   // bytes 4 kb .. 4 kb + 3
             q[k] = deq4x4((part & 2 ? w >> 4 : w) & 0x0f0f0f0fu, dd);
         }
-        *reinterpret_cast<u4 *>(tile + key * stride + b * 64 + part * 16) = u4{q[0].lo, q[0].hi, q[1].lo, q[1].hi};
+        *reinterpret_cast<u4 *>(tile + pf_lay<D>::key_off(key, stride) + b * 64 + part * 16) = u4{q[0].lo, q[0].hi, q[1].lo, q[1].hi};
     }
 };
 
@@ -186,9 +208,17 @@ template <class S> __device__ __forceinline__ void store_tile(const typename S::
 }
 
 // GROUPED: pages hold at least 16 positions (or the cache is contiguous), so a 16-key group has one base
-template <uint32_t KT, int D, bool GROUPED>
+__device__ __forceinline__ uint32_t lds_addr(const char * p) { return (uint32_t) (size_t) (const __attribute__((address_space(3))) char *) p; }
+// 64 lanes x 16 bytes, global (scalar base + 32-bit lane offset) -> LDS at `lds` + 16 * lane, no registers in between
+__device__ __forceinline__ void dma16(const char * sbase, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+}
+
+template <uint32_t KT, int D, bool GROUPED, bool DMA>
 __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
+    static_assert(!DMA || (KT == P1A_KV_F16 && GROUPED && D == 256), "the LDS-direct loads are laid out for f16 rows of 512 bytes");
     using C = pf_cfg<D>;
+    using L = pf_lay<D>;
     using S = stager<KT, D>;
     extern __shared__ __attribute__((aligned(16))) char lds[];
 
@@ -228,18 +258,35 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             const float s = P.qscale;
             qf[ks] = h8{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s),
                         (half_t) (b.x * s), (half_t) (b.y * s), (half_t) (b.z * s), (half_t) (b.w * s)};
+            // Q stays in accumulation registers for the whole kernel: the matrix instructions read them in place, and
+            // the vector registers are left to the tiles in flight
+            asm volatile("" : "+a"(qf[ks]));
         }
     }
 
-    f16x o[C::NDT];
-    f16x ol;
+    // Waves pair up for O^T: the pair (w, w ^ 1) shares its 64 query rows, each wave accumulating HALF the dims
+    // (tiles HD * (w & 1) ..) for ALL 64 rows: a V^T fragment read from LDS then feeds two MFMAs (own rows, partner's
+    // rows) instead of one, which halves the transposing reads - the slowest LDS traffic of the kernel. The price is
+    // that P^T (and the rare rescale factors) of the partner come through LDS, behind one more barrier per tile.
+    constexpr int HD = C::NDT / 2;                            // dim tiles per wave
+    static_assert(C::NDT % 2 == 0, "the dims split over a pair of waves");
+    const int dh = wave & 1;                                  // which half of the dims
+    f16x o[2][HD];                                            // [0]: own rows, [1]: the partner's rows
+    f16x ol;                                                  // softmax denominator of the own rows
     float m_run = NEG_INF;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         ol[i] = 0.f;
 #pragma unroll
-        for (int dt = 0; dt < C::NDT; ++dt) o[dt][i] = 0.f;
+        for (int dt = 0; dt < HD; ++dt) { o[0][dt][i] = 0.f; o[1][dt][i] = 0.f; }
     }
+    // exchange areas behind the tile stages: P^T of every wave (BN / 16 k-steps x 64 lanes x 16 bytes), then one float
+    // per query row (rescale factor during the loop, denominator at the end)
+    char * const xbase = lds + 2 * L::STAGE_B + (S::SCALES_VIA_LDS ? 2 * 4 * 16 * S::SB : 0);
+    constexpr int PX_B = (BN / 16) * 64 * 16;
+    char * const px_own = xbase + wave * PX_B, * const px_par = xbase + (wave ^ 1) * PX_B;
+    float * const ax_own = reinterpret_cast<float *>(xbase + 4 * PX_B) + wave * 32;
+    float * const ax_par = reinterpret_cast<float *>(xbase + 4 * PX_B) + (wave ^ 1) * 32;
     const h8 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
 
     // ---- addressing of the raw tile ----
@@ -324,7 +371,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     const int lkey = 16 * wave + l16;
     const uint32_t sb_full = (uint32_t) l16 * (uint32_t) P.pg.rowb;
     const uint32_t sb_last = (uint32_t) min(l16, max(pmax - (last_tile * BN + 16 * wave), 0)) * (uint32_t) P.pg.rowb;
-    char * const ksc = lds + 2 * C::STAGE_B + wave * 16 * S::SB;           // this wave's parking area: K blocks
+    char * const ksc = lds + 2 * L::STAGE_B + wave * 16 * S::SB;           // this wave's parking area: K blocks
     char * const vsc = ksc + 4 * 16 * S::SB;                               // ... V blocks
     auto load_sblk = [&](const char * cache, int tile, const gbases & gb) {
         sblk r;
@@ -374,7 +421,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         for (int u = 0; u < 2; ++u) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) s[u][i] = 0.f;
-            const char * krow = kt + (32 * u + c) * C::KSTR + g * 16;
+            const char * krow = kt + L::k_lane(c) + L::k_half(u) + g * 16;
 #pragma unroll
             for (int ks = 0; ks < C::NKS; ++ks) {
                 const h8 a = *reinterpret_cast<const h8 *>(krow + ks * 32);
@@ -383,20 +430,46 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         }
     };
 
-    // ---- prologue: K(0), V(0), K(1) in LDS; V(1) and K(2) on their way in registers; S^T(0) ----
+    // ---- LDS-direct tile loads (DMA): wave w moves the 8 blocks of its 16-key group; instruction j takes keys j and
+    // j + 8 of the group (lanes 0-31 / 32-63, 16 bytes of the row each). In the tile that holds pmax the rows past it
+    // repeat the last written one ----
+    // (no branches: the two row numbers of a block are clamped in scalar registers, each lane picks its own)
+    const uint32_t dma_col = (uint32_t) (lane & 31) * 16u;
+    const int dma_room = __builtin_amdgcn_readfirstlane(max(pmax - (last_tile * BN + 16 * wave), 0));
+    auto dma_block = [&](const char * cache, int tile, const gbases & gb, char * dst_tile, int bstride, int j) {
+        const int room = tile == last_tile ? dma_room : 15;
+        const uint32_t r0 = __builtin_amdgcn_readfirstlane((uint32_t) min(j, room) * (uint32_t) P.pg.rowb);
+        const uint32_t r1 = __builtin_amdgcn_readfirstlane((uint32_t) min(j + 8, room) * (uint32_t) P.pg.rowb);
+        dma16(cache + gb.go, (g ? r1 : r0) + dma_col, lds_addr(dst_tile + (8 * wave + j) * bstride));
+    };
+
+    // ---- prologue: K(0), V(0), K(1) in LDS; (staged through registers: V(1) and K(2) on their way); S^T(0) ----
     typename S::raw rk, rv;
     sblk sk, sv;                                           // scale blocks that belong to rk, rv
     gbases gb_prev;                                        // group bases of the tile whose V is fetched next
-    {
+    gpages gp_ahead;                                       // (DMA) table entry of the K tile fetched in the next step
+    if constexpr (DMA) {
+        gpages g0 = group_pages(tile_of(0)), g1 = group_pages(tile_of(1));
+        const gbases b0 = group_bases(tile_of(0), g0);
+        gb_prev = group_bases(tile_of(1), g1);
+        gp_ahead = group_pages(tile_of(2));
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dma_block(P.kc, tile_of(0), b0, lds, L::KB, j);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dma_block(P.vc, tile_of(0), b0, lds + L::KT_B, L::VB, j);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dma_block(P.kc, tile_of(1), gb_prev, lds + L::STAGE_B, L::KB, j);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    } else {
         gpages g0 = group_pages(tile_of(0)), g1 = group_pages(tile_of(1)), g2 = group_pages(tile_of(2));
         const gbases b0 = group_bases(tile_of(0), g0), b1 = group_bases(tile_of(1), g1);
         gb_prev = group_bases(tile_of(2), g2);
         fetch_tile(rk, P.kc, ksc, tile_of(0), b0);
         fetch_tile(rv, P.vc, vsc, tile_of(0), b0);
-        store_tile<S>(rk, lds, C::KSTR, tid);
-        store_tile<S>(rv, lds + C::KT_B, C::VSTR, tid);
+        store_tile<S>(rk, lds, L::KB, tid);
+        store_tile<S>(rv, lds + L::KT_B, L::VB, tid);
         fetch_tile(rk, P.kc, ksc, tile_of(1), b1);
-        store_tile<S>(rk, lds + C::STAGE_B, C::KSTR, tid);
+        store_tile<S>(rk, lds + L::STAGE_B, L::KB, tid);
         load_tile(rv, P.vc, tile_of(1), b1);
         load_tile(rk, P.kc, tile_of(2), gb_prev);
         if constexpr (SVL) { sv = load_sblk(P.vc, tile_of(1), b1); sk = load_sblk(P.kc, tile_of(2), gb_prev); }
@@ -404,6 +477,8 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     __syncthreads();
     f16x s_next[2];
     qk(lds, s_next);
+    // (the first step overwrites K(0) while it runs; every wave has to be done reading it)
+    if constexpr (DMA) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
 #ifdef P1A_TRACE
     long long acc_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -411,9 +486,14 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 #endif
     for (int it = 0; it < ntiles; ++it) {
         const int k0 = tile_of(it) * BN;
-        char * const st_cur = lds + (it & 1) * C::STAGE_B;             // holds K(it) (done with) and V(it)
-        char * const st_nxt = lds + ((it + 1) & 1) * C::STAGE_B;       // holds K(it+1); V(it-1) is done with
-        gpages gp_k = group_pages(tile_of(it + 3));                    // entries for the K fetch at the end of this step
+        char * const st_cur = lds + (it & 1) * L::STAGE_B;             // holds K(it) (done with) and V(it)
+        char * const st_nxt = lds + ((it + 1) & 1) * L::STAGE_B;       // holds K(it+1); V(it-1) is done with
+        gpages gp_k;
+        gbases gb_dma;
+        if constexpr (DMA) {
+            gb_dma = group_bases(tile_of(it + 2), gp_ahead);           // K(it+2) goes over K(it), V(it+1) over V(it-1):
+            gp_ahead = group_pages(tile_of(it + 3));                   // requested between the S^T steps below
+        } else gp_k = group_pages(tile_of(it + 3));                    // entries for the K fetch at the end of this step
         f16x s[2] = {s_next[0], s_next[1]};
 
         // ---- stream 1: S^T(it+1) on the matrix pipe; stream 2: softmax of S^T(it) on the vector pipe ----
@@ -423,12 +503,19 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         h8 pb[BN / 16];
         constexpr int NQK = 2 * C::NKS, HALF = NQK / 2, VPS = 32 / HALF, PF_K = 4;
         static_assert(32 % HALF == 0 && (8 % VPS == 0 || VPS % 8 == 0), "softmax slices must tile the 32 values of a lane");
-        // this lane holds keys k0 + 32 u + 8 (i / 4) + 4 g + (i % 4) of its own row
+        // this lane holds keys k0 + key_of(u, i) + 4 g of its own row
         const int lim = my_pos - k0 - 4 * g;
-        const char * krow = st_nxt + c * C::KSTR + g * 16;
-        auto kfrag = [&](int k) { return *reinterpret_cast<const h8 *>(krow + (k / C::NKS) * 32 * C::KSTR + (k % C::NKS) * 32); };
+        const char * krow = st_nxt + L::k_lane(c) + g * 16;
+        auto kfrag = [&](int k) { return *reinterpret_cast<const h8 *>(krow + L::k_half(k / C::NKS) + (k % C::NKS) * 32); };
         auto qk_step = [&](h8 (&fr)[NQK], int k) {
             if (k + PF_K < NQK) fr[k + PF_K] = kfrag(k + PF_K);
+            if constexpr (DMA) {   // one tile load every other step: K(it+2) first (it is needed first), then V(it+1)
+                if (k % 2 == 0) {
+                    const int j = k / 2;
+                    if (j < 8) dma_block(P.kc, tile_of(it + 2), gb_dma, st_cur, L::KB, j);
+                    else if (j < 16) dma_block(P.vc, tile_of(it + 1), gb_prev, st_nxt + L::KT_B, L::VB, j - 8);
+                }
+            }
             const int u = k / C::NKS;
             if (k % C::NKS == 0) {
 #pragma unroll
@@ -446,7 +533,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 #pragma unroll
             for (int v = 0; v < VPS; ++v) {
                 const int idx = k * VPS + v, su = idx >> 4, i = idx & 15;
-                s[su][i] = 32 * su + 8 * (i >> 2) + (i & 3) <= lim ? s[su][i] : NEG_INF;
+                s[su][i] = L::key_of(su, i) <= lim ? s[su][i] : NEG_INF;
                 mloc = fmaxf(mloc, s[su][i]);
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -462,6 +549,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         const bool dead = mnew == NEG_INF;
         const float alpha = (fresh || mnew == m_run) ? 1.0f : __builtin_amdgcn_exp2f(m_run - mnew);
         m_run = mnew;
+        const float msub = dead ? 0.0f : mnew;                       // a row with no visible key yet: exp2(-inf - 0) = 0
         // (the branch sits in the middle of the S^T products on purpose: what follows it runs straight into the O^T
         // products, so P is formed in the shadow of the remaining S^T MFMAs instead of being sunk to its first use)
         if (__builtin_expect(__any(alpha != 1.0f), 0)) {
@@ -469,7 +557,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             for (int i = 0; i < 16; ++i) {
                 ol[i] *= alpha;
 #pragma unroll
-                for (int dt = 0; dt < C::NDT; ++dt) o[dt][i] *= alpha;
+                for (int dt = 0; dt < HD; ++dt) o[0][dt][i] *= alpha;
             }
         }
         PT(1);
@@ -483,51 +571,67 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 #pragma unroll
             for (int v = 0; v < VPS; ++v) {
                 const int idx = (k - HALF) * VPS + v, su = idx >> 4, i = idx & 15;
-                s[su][i] = dead ? 0.0f : __builtin_amdgcn_exp2f(s[su][i] - mnew);
-                if ((idx & 7) == 7) {
-                    const int b = i - 7;
-                    pb[idx >> 3] = h8{(half_t) s[su][b], (half_t) s[su][b + 1], (half_t) s[su][b + 2], (half_t) s[su][b + 3],
-                                      (half_t) s[su][b + 4], (half_t) s[su][b + 5], (half_t) s[su][b + 6], (half_t) s[su][b + 7]};
+                s[su][i] = __builtin_amdgcn_exp2f(s[su][i] - msub);
+                if (idx & 1) {   // packed conversion (round to nearest even), two values per instruction
+                    const h2 pr = __builtin_convertvector(f2v{s[su][i - 1], s[su][i]}, h2);
+                    pb[idx >> 3][(idx & 7) - 1] = pr[0];
+                    pb[idx >> 3][idx & 7] = pr[1];
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
 
         PT(2);
+        // ---- hand P^T and the rescale factor of the own rows to the partner ----
+#pragma unroll
+        for (int ps = 0; ps < BN / 16; ++ps) *reinterpret_cast<h8 *>(px_own + (ps * 64 + lane) * 16) = pb[ps];
+        if (g == 0) ax_own[c] = alpha;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        {
+            const float alpha_p = ax_par[c];
+            if (__builtin_expect(__any(alpha_p != 1.0f), 0)) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+#pragma unroll
+                    for (int dt = 0; dt < HD; ++dt) o[1][dt][i] *= alpha_p;
+            }
+        }
+        PT(6);
         // ---- stream 1: O^T += V^T(it) P^T on the matrix pipe; stream 2: K(it+2), V(it+1) -> f16 tiles in LDS ----
         {
-            // Slot e of lane half g in k-step ps is key 16 ps + 4 g + e (e < 4) or 16 ps + 8 + 4 g + e - 4
+            // Slot e of lane half g in k-step ps is key 32 (ps / 2) + 8 (ps % 2) + 4 g + e (e < 4), or that + 16 for e - 4
             const int i16 = lane & 15, blk = lane >> 4;        // 16-lane block: dims 16 (blk & 1) .., lane half blk >> 1 == g
             const int kk = i16 >> 2, jq = i16 & 3;
-            const char * vbase = st_cur + C::KT_B + (4 * g + kk) * C::VSTR + (16 * (blk & 1) + 4 * jq) * 2;
-            constexpr int NMF = C::NDT + 1, NPV = (BN / 16) * NMF, PF_V = 3;      // per k-step: NDT tiles of O^T, then the ones
+            const char * vbase = st_cur + L::KT_B + L::v_lane(4 * g + kk) + (16 * (blk & 1) + 4 * jq) * 2 + dh * HD * 64;
+            // per k-step: HD fragments of V^T, each multiplied with the own and the partner's P^T, then the denominator
+            constexpr int NFR = (BN / 16) * HD, PF_V = 3;
             constexpr int NP = 2 * S::NPT * S::PARTS;                             // store parts: K items, then V items
             struct vfrag { s4 lo, hi; };
-            auto vread = [&](int k) {
-                const char * p0_ = vbase + (16 * (k / NMF)) * C::VSTR + (k % NMF) * 64;
-                return vfrag{__builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) p0_),
-                             __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + 8 * C::VSTR))};
+            auto vread = [&](int f) {
+                const char * p0_ = vbase + (f % HD) * 64;
+                return vfrag{__builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + L::v_lo(f / HD))),
+                             __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + L::v_hi(f / HD)))};
             };
-            vfrag vf[NPV];
+            vfrag vf[NFR];
+            h8 pp[BN / 16];
 #pragma unroll
-            for (int k = 0; k < PF_V; ++k)
-                if (k % NMF != C::NDT) vf[k] = vread(k);
+            for (int f = 0; f < PF_V && f < NFR; ++f) vf[f] = vread(f);
+            pp[0] = *reinterpret_cast<const h8 *>(px_par + lane * 16);
 #pragma unroll
-            for (int k = 0; k < NPV; ++k) {
-                if (k + PF_V < NPV && (k + PF_V) % NMF != C::NDT) vf[k + PF_V] = vread(k + PF_V);
-                const int ps = k / NMF, dt = k % NMF;
-                if (dt < C::NDT) {
-                    const h4 l4 = __builtin_bit_cast(h4, vf[k].lo), h4_ = __builtin_bit_cast(h4, vf[k].hi);
-                    const h8 a = {l4[0], l4[1], l4[2], l4[3], h4_[0], h4_[1], h4_[2], h4_[3]};
-                    o[dt < C::NDT ? dt : 0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[ps], o[dt < C::NDT ? dt : 0], 0, 0, 0);
-                } else {
-                    ol = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[ps], ol, 0, 0, 0);
-                }
+            for (int f = 0; f < NFR; ++f) {
+                if (f + PF_V < NFR) vf[f + PF_V] = vread(f + PF_V);
+                const int ps = f / HD, dt = f % HD;
+                if (dt == 0 && ps + 1 < BN / 16) pp[ps + 1] = *reinterpret_cast<const h8 *>(px_par + ((ps + 1) * 64 + lane) * 16);
+                const h4 l4 = __builtin_bit_cast(h4, vf[f].lo), h4_ = __builtin_bit_cast(h4, vf[f].hi);
+                const h8 a = {l4[0], l4[1], l4[2], l4[3], h4_[0], h4_[1], h4_[2], h4_[3]};
+                o[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[ps], o[0][dt], 0, 0, 0);
+                o[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pp[ps], o[1][dt], 0, 0, 0);
+                if (dt == HD - 1) ol = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[ps], ol, 0, 0, 0);
 #pragma unroll
-                for (int pt = k * NP / NPV; pt < (k + 1) * NP / NPV; ++pt) {
+                for (int pt = DMA ? NP : f * NP / NFR; pt < (f + 1) * NP / NFR; ++pt) {
                     const int item = pt / S::PARTS, part = pt % S::PARTS;
-                    if (item < S::NPT) S::store_part(rk, st_cur, C::KSTR, tid, item, part);                          // K(it+2) over K(it)
-                    else               S::store_part(rv, st_nxt + C::KT_B, C::VSTR, tid, item - S::NPT, part);       // V(it+1) over V(it-1)
+                    if (item < S::NPT) S::store_part(rk, st_cur, L::KB, tid, item, part);                          // K(it+2) over K(it)
+                    else               S::store_part(rv, st_nxt + L::KT_B, L::VB, tid, item - S::NPT, part);       // V(it+1) over V(it-1)
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -536,7 +640,10 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         PT(3);
         // ---- raw loads of K(it+3), V(it+2): one whole step to arrive. Issued back to back: a vector memory instruction
         // holds the wave for as long as the CU's address path needs for it, wherever it is placed ----
-        {
+        if constexpr (DMA) {
+            gb_prev = gb_dma;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this step's tile loads have landed
+        } else {
             const gbases gb_k = group_bases(tile_of(it + 3), gp_k);
             load_tile(rk, P.kc, tile_of(it + 3), gb_k);
             load_tile(rv, P.vc, tile_of(it + 2), gb_prev);
@@ -552,34 +659,41 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 #ifdef P1A_TRACE
     if (g_pf_trace && tid == 0) for (int i = 0; i < 8; ++i) g_pf_trace[(size_t) blockIdx.x * 8 + i] = acc_t[i];
 #endif
-    // ---- epilogue: normalise, gate, store. Lane (row c, half g) holds dims 32 dt + 8 (i / 4) + 4 g + (i % 4) ----
-    if (live) {
-        const float inv = 1.0f / ol[0];
-        float * orow = P.out + ((size_t) my_tok * P.Hq + h) * D;
-        const float * grow = P.gate ? P.gate + ((size_t) my_tok * P.Hq + h) * D : nullptr;
+    // ---- epilogue: the pair swaps denominators, then each wave normalises, gates and stores its half of the dims of
+    // all 64 rows. Lane (row c, half g) holds dims 32 dt + 8 (i / 4) + 4 g + (i % 4) of tile dt ----
+    if (g == 0) ax_own[c] = ol[0];
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // (also: no tile load is left in flight)
+    const float l_par = ax_par[c];
 #pragma unroll
-        for (int dt = 0; dt < C::NDT; ++dt)
+    for (int r = 0; r < 2; ++r) {
+        const int tok = tok0 + 32 * (r ? wave ^ 1 : wave) + c;
+        if (tok >= P.T) continue;
+        const float inv = 1.0f / (r ? l_par : ol[0]);
+        float * orow = P.out + ((size_t) tok * P.Hq + h) * D;
+        const float * grow = P.gate ? P.gate + ((size_t) tok * P.Hq + h) * D : nullptr;
+#pragma unroll
+        for (int dt = 0; dt < HD; ++dt)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
-                const int d0 = 32 * dt + 8 * q4 + 4 * g;
-                f4 r = {o[dt][4 * q4] * inv, o[dt][4 * q4 + 1] * inv, o[dt][4 * q4 + 2] * inv, o[dt][4 * q4 + 3] * inv};
+                const int d0 = 32 * (dh * HD + dt) + 8 * q4 + 4 * g;
+                f4 rr = {o[r][dt][4 * q4] * inv, o[r][dt][4 * q4 + 1] * inv, o[r][dt][4 * q4 + 2] * inv, o[r][dt][4 * q4 + 3] * inv};
                 if (grow) {
                     const f4 gt = *reinterpret_cast<const f4 *>(grow + d0);
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) r[x] *= 1.0f / (1.0f + expf(-gt[x]));
+                    for (int x = 0; x < 4; ++x) rr[x] *= 1.0f / (1.0f + expf(-gt[x]));
                 }
-                *reinterpret_cast<f4 *>(orow + d0) = r;
+                *reinterpret_cast<f4 *>(orow + d0) = rr;
             }
     }
 }
 
-template <uint32_t KT, int D, bool GROUPED>
+template <uint32_t KT, int D, bool GROUPED, bool DMA = false>
 int launch_pf_g(const pf_params & P, hipStream_t s) {
-    using C = pf_cfg<D>;
-    const int lds = 2 * C::STAGE_B + (stager<KT, D>::SCALES_VIA_LDS ? 2 * 4 * 16 * stager<KT, D>::SB : 0);
+    using L = pf_lay<D>;
+    const int lds = 2 * L::STAGE_B + (stager<KT, D>::SCALES_VIA_LDS ? 2 * 4 * 16 * stager<KT, D>::SB : 0) + 4 * (BN / 16) * 64 * 16 + 4 * 32 * 4;
     static bool attr_set = false;
     if (!attr_set) {
-        if (hipFuncSetAttribute((const void *) prefill_k<KT, D, GROUPED>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+        if (hipFuncSetAttribute((const void *) prefill_k<KT, D, GROUPED, DMA>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
             (void) hipGetLastError();
             set_error("p1a_attn_prefill: cannot reserve %d bytes of LDS", lds);
             return P1A_E_LAUNCH;
@@ -588,12 +702,18 @@ int launch_pf_g(const pf_params & P, hipStream_t s) {
     }
     const int units = P.nblk * P.Hkv;
     const int slots = ((units + 7) / 8) * P.GQA;
-    prefill_k<KT, D, GROUPED><<<slots * 8, NTHR, lds, s>>>(P);
+    prefill_k<KT, D, GROUPED, DMA><<<slots * 8, NTHR, lds, s>>>(P);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 template <uint32_t KT, int D>
 int launch_pf(const pf_params & P, hipStream_t s) {
-    return !P.pg.pt || P.pg.psh >= 4 ? launch_pf_g<KT, D, true>(P, s) : launch_pf_g<KT, D, false>(P, s);
+    const bool grouped = !P.pg.pt || P.pg.psh >= 4;
+    if constexpr (KT == P1A_KV_F16 && D == 256) {
+        static const bool no_dma = getenv("P1A_PF_NODMA") && atoi(getenv("P1A_PF_NODMA"));   // development A/B switch
+        // (rows of whole 16-byte units at 16-byte aligned addresses: what a 16-byte load per lane needs)
+        if (grouped && !no_dma && P.pg.rowb % 16 == 0 && P.pg.rowb * 16 < (1ull << 32)) return launch_pf_g<KT, D, true, true>(P, s);
+    }
+    return grouped ? launch_pf_g<KT, D, true>(P, s) : launch_pf_g<KT, D, false>(P, s);
 }
 
 }   // namespace
