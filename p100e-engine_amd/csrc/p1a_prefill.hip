@@ -477,6 +477,22 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     __syncthreads();
     f16x s_next[2];
     qk(lds, s_next);
+    // Masking and the row maximum of a tile are done one step ahead of its softmax (in the shadow of the O^T products of
+    // the tile before it): value i of half u of a lane's S^T column is key k0 + key_of(u, i) + 4 g of the lane's own row.
+    auto mask_max = [&](f16x (&sv_)[2], int k0_, int idx, float m) {
+        const int su = idx >> 4, i = idx & 15;
+        sv_[su][i] = L::key_of(su, i) <= my_pos - k0_ - 4 * g ? sv_[su][i] : NEG_INF;
+        return fmaxf(m, sv_[su][i]);
+    };
+    // both lane halves of a row -> the row's maximum
+    auto row_max = [&](float m) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, m), __builtin_bit_cast(unsigned, m), false, false);
+        return fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+    };
+    float mloc = NEG_INF;
+#pragma unroll
+    for (int idx = 0; idx < 32; ++idx) mloc = mask_max(s_next, tile_of(0) * BN, idx, mloc);
+    mloc = row_max(mloc);
     // (the first step overwrites K(0) while it runs; every wave has to be done reading it)
     if constexpr (DMA) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
@@ -494,20 +510,41 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             gb_dma = group_bases(tile_of(it + 2), gp_ahead);           // K(it+2) goes over K(it), V(it+1) over V(it-1):
             gp_ahead = group_pages(tile_of(it + 3));                   // requested between the S^T steps below
         } else gp_k = group_pages(tile_of(it + 3));                    // entries for the K fetch at the end of this step
-        f16x s[2] = {s_next[0], s_next[1]};
+        f16x s[2] = {s_next[0], s_next[1]};                            // S^T(it), masked; mloc = its row maximum
 
-        // ---- stream 1: S^T(it+1) on the matrix pipe; stream 2: softmax of S^T(it) on the vector pipe ----
+        // Lazy reference maximum: m_run follows the row maximum only when it has grown by more than RESCALE_STEP, so P
+        // stays below 2^RESCALE_STEP (well inside f16) and the accumulators are rescaled a handful of times per row
+        // instead of at every tile. A row that has seen no visible key yet (m_run = -inf) just adopts the maximum.
+        const bool fresh = m_run == NEG_INF;
+        const bool move = mloc > m_run + RESCALE_STEP || fresh;      // mloc = -inf never moves anything
+        const float mnew = (move && mloc != NEG_INF) ? mloc : m_run;
+        const bool dead = mnew == NEG_INF;
+        const float alpha = (fresh || mnew == m_run) ? 1.0f : __builtin_amdgcn_exp2f(m_run - mnew);
+        m_run = mnew;
+        const float msub = dead ? 0.0f : mnew;                       // a row with no visible key yet: exp2(-inf - 0) = 0
+        if (__builtin_expect(__any(alpha != 1.0f), 0)) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                ol[i] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < HD; ++dt) o[0][dt][i] *= alpha;
+            }
+        }
+        PT(0);
+
+        // ---- stream 1: S^T(it+1) on the matrix pipe; stream 2: P^T(it) = exp2(S^T(it) - m) on the vector pipe ----
         // Written step by step, one MFMA per step, with a scheduling fence after each: the LDS read of the K fragment
-        // PF_K steps ahead, the MFMA, and a slice of the softmax that fits in the MFMA's shadow. The first half of the
-        // steps masks and finds the row maximum, the middle one settles the reference maximum, the second half forms P.
+        // PF_K steps ahead, the MFMA, and a slice of the softmax that fits in the MFMA's shadow.
         h8 pb[BN / 16];
-        constexpr int NQK = 2 * C::NKS, HALF = NQK / 2, VPS = 32 / HALF, PF_K = 4;
-        static_assert(32 % HALF == 0 && (8 % VPS == 0 || VPS % 8 == 0), "softmax slices must tile the 32 values of a lane");
-        // this lane holds keys k0 + key_of(u, i) + 4 g of its own row
-        const int lim = my_pos - k0 - 4 * g;
+        constexpr int NQK = 2 * C::NKS, VPS = 32 / NQK, PF_K = 4;
+        static_assert(32 % NQK == 0 && (VPS == 1 || VPS % 2 == 0), "softmax slices must tile the 32 values of a lane");
         const char * krow = st_nxt + L::k_lane(c) + g * 16;
         auto kfrag = [&](int k) { return *reinterpret_cast<const h8 *>(krow + L::k_half(k / C::NKS) + (k % C::NKS) * 32); };
-        auto qk_step = [&](h8 (&fr)[NQK], int k) {
+        h8 fr[NQK];
+#pragma unroll
+        for (int k = 0; k < PF_K; ++k) fr[k] = kfrag(k);
+#pragma unroll
+        for (int k = 0; k < NQK; ++k) {
             if (k + PF_K < NQK) fr[k + PF_K] = kfrag(k + PF_K);
             if constexpr (DMA) {   // one tile load every other step: K(it+2) first (it is needed first), then V(it+1)
                 if (k % 2 == 0) {
@@ -522,55 +559,13 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                 for (int i = 0; i < 16; ++i) s_next[u][i] = 0.f;
             }
             s_next[u] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fr[k], qf[k % C::NKS], s_next[u], 0, 0, 0);
-        };
-        h8 fr[NQK];
-#pragma unroll
-        for (int k = 0; k < PF_K; ++k) fr[k] = kfrag(k);
-        float mloc = NEG_INF;
-#pragma unroll
-        for (int k = 0; k < HALF; ++k) {
-            qk_step(fr, k);
-#pragma unroll
-            for (int v = 0; v < VPS; ++v) {
-                const int idx = k * VPS + v, su = idx >> 4, i = idx & 15;
-                s[su][i] = L::key_of(su, i) <= lim ? s[su][i] : NEG_INF;
-                mloc = fmaxf(mloc, s[su][i]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        PT(0);
-        mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-        // Lazy reference maximum: m_run follows the row maximum only when it has grown by more than RESCALE_STEP, so P
-        // stays below 2^RESCALE_STEP (well inside f16) and the accumulators are rescaled a handful of times per row
-        // instead of at every tile. A row that has seen no visible key yet (m_run = -inf) just adopts the maximum.
-        const bool fresh = m_run == NEG_INF;
-        const bool move = mloc > m_run + RESCALE_STEP || fresh;      // mloc = -inf never moves anything
-        const float mnew = (move && mloc != NEG_INF) ? mloc : m_run;
-        const bool dead = mnew == NEG_INF;
-        const float alpha = (fresh || mnew == m_run) ? 1.0f : __builtin_amdgcn_exp2f(m_run - mnew);
-        m_run = mnew;
-        const float msub = dead ? 0.0f : mnew;                       // a row with no visible key yet: exp2(-inf - 0) = 0
-        // (the branch sits in the middle of the S^T products on purpose: what follows it runs straight into the O^T
-        // products, so P is formed in the shadow of the remaining S^T MFMAs instead of being sunk to its first use)
-        if (__builtin_expect(__any(alpha != 1.0f), 0)) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                ol[i] *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < HD; ++dt) o[0][dt][i] *= alpha;
-            }
-        }
-        PT(1);
-#pragma unroll
-        for (int k = HALF; k < NQK; ++k) {
-            qk_step(fr, k);
             if constexpr (SVL) {   // the scales of the raw tiles fetched one step ago: through LDS to the lanes that use them
                 if (k == NQK - 4) { park_sblk(ksc, sk); park_sblk(vsc, sv); }
                 if (k == NQK - 2) { pick_scales(rk, ksc); pick_scales(rv, vsc); }
             }
 #pragma unroll
             for (int v = 0; v < VPS; ++v) {
-                const int idx = (k - HALF) * VPS + v, su = idx >> 4, i = idx & 15;
+                const int idx = k * VPS + v, su = idx >> 4, i = idx & 15;
                 s[su][i] = __builtin_amdgcn_exp2f(s[su][i] - msub);
                 if (idx & 1) {   // packed conversion (round to nearest even), two values per instruction
                     const h2 pr = __builtin_convertvector(f2v{s[su][i - 1], s[su][i]}, h2);
@@ -614,6 +609,10 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             };
             vfrag vf[NFR];
             h8 pp[BN / 16];
+            constexpr int MPS = 32 / NFR;                                          // next tile's values masked per step
+            static_assert(32 % NFR == 0, "mask slices must tile the 32 values of a lane");
+            const int k0n = tile_of(it + 1) * BN;
+            mloc = NEG_INF;
 #pragma unroll
             for (int f = 0; f < PF_V && f < NFR; ++f) vf[f] = vread(f);
             pp[0] = *reinterpret_cast<const h8 *>(px_par + lane * 16);
@@ -628,6 +627,8 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                 o[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pp[ps], o[1][dt], 0, 0, 0);
                 if (dt == HD - 1) ol = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[ps], ol, 0, 0, 0);
 #pragma unroll
+                for (int v = 0; v < MPS; ++v) mloc = mask_max(s_next, k0n, f * MPS + v, mloc);
+#pragma unroll
                 for (int pt = DMA ? NP : f * NP / NFR; pt < (f + 1) * NP / NFR; ++pt) {
                     const int item = pt / S::PARTS, part = pt % S::PARTS;
                     if (item < S::NPT) S::store_part(rk, st_cur, L::KB, tid, item, part);                          // K(it+2) over K(it)
@@ -637,6 +638,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             }
         }
 
+        mloc = row_max(mloc);
         PT(3);
         // ---- raw loads of K(it+3), V(it+2): one whole step to arrive. Issued back to back: a vector memory instruction
         // holds the wave for as long as the CU's address path needs for it, wherever it is placed ----
