@@ -1,16 +1,20 @@
 // Chunked causal prefill attention over a paged f16 / q8_0 / q4_0 KV cache for gfx950 (MI355X).
 //
 // One workgroup (4 waves, one per SIMD, 512 registers each) owns 128 consecutive query tokens of ONE q head; wave w owns
-// 32 of them as the N = 32 columns of v_mfma_f32_32x32x16_f16 tiles. Keys are walked in tiles of 64: all 256 threads
-// fetch the raw tile of the head's kv head (16-byte loads off a wave-uniform page base), dequantize it in registers and
-// store it to LDS as f16 [key][dim] (two K and two V buffers, one barrier per tile).
-//   S^T = K Q^T : A = K rows straight from LDS (ds_read_b128), B = Q^T held in registers (pre-multiplied by
-//                 scale * log2 e, rounded to f16). A lane then holds 16 keys of ONE query row, so the row maximum
+// 32 of them as the N = 32 columns of v_mfma_f32_32x32x16_f16 tiles. Keys are walked in tiles of 64, kept in LDS as f16
+// (two K and two V tiles). f16 rows of 512 bytes are moved from global memory straight into LDS
+// (global_load_lds_dwordx4); everything else is fetched into registers with 16-byte loads off a wave-uniform page base,
+// dequantized and stored to the same LDS places.
+//   S^T = K Q^T : A = K rows straight from LDS (ds_read_b128), B = Q^T held in accumulation registers (pre-multiplied
+//                 by scale * log2 e, rounded to f16). A lane then holds 16 keys of ONE query row, so the row maximum
 //                 needs no cross-lane work beyond one half-wave swap.
 //   O^T = V^T P^T : A = V^T read with the transposing ds_read_b64_tr_b16, B = P^T straight from the S^T registers.
+//                 Waves pair up: each wave of a pair accumulates half the dims for the 64 rows of both, so a V^T
+//                 fragment feeds two MFMAs; the partner's P^T comes through LDS.
 // The loop is software-pipelined so that every iteration holds two independent instruction streams side by side: the
-// MFMAs of S^T for tile j+1 next to the softmax VALU work of tile j, then the MFMAs of O^T for tile j next to the
-// dequantization of the tiles that come after. With one wave per SIMD nothing else can hide one pipe behind the other.
+// MFMAs of S^T for tile j+1 next to exp2 / f16 conversion of tile j, then the MFMAs of O^T for tile j next to masking and
+// the row maximum of tile j+1 (and the dequantization of the tiles that come after). With one wave per SIMD nothing
+// else can hide one pipe behind the other.
 // fp32 accumulation; the softmax denominator is accumulated by an MFMA against an all-ones operand so that it sums the
 // same rounded P that multiplies V. The reference maximum of a row moves lazily (only when the row maximum has grown
 // by more than 2^RESCALE_STEP), so the accumulators are rescaled a handful of times per row. Keys above a row's
