@@ -36,6 +36,8 @@ extern "C" {
 #define P1A_E_ARG        (-2) /* null or inconsistent argument */
 #define P1A_E_SCRATCH    (-3) /* scratch allocation failed or caller scratch too small */
 #define P1A_E_LAUNCH     (-4) /* the HIP runtime reported a launch error */
+#define P1A_E_STATE      (-5) /* pool / sequence manager: the pool or the sequence is not in a state that allows it */
+#define P1A_E_IO         (-6) /* session file: cannot open, short read / write, or not a loadable file */
 
 #define P1A_MAX_ROWS 32 /* query rows per p1a_attn_decode call (the reference allows 8: src/fast/attn.cuh:66) */
 

@@ -10,6 +10,13 @@ EXPORTS = [
     "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_release", "p1a_last_error",
     "p1a_version",
+    # include/p1a_pool.h
+    "p1a_pool_create", "p1a_pool_destroy", "p1a_pool_n_pages", "p1a_pool_free_pages", "p1a_pool_max_pages", "p1a_pool_page_bytes",
+    "p1a_pool_host_used", "p1a_pool_kv_seq", "p1a_pool_kv_rows", "p1a_pool_set_rows", "p1a_pool_state", "p1a_seq_create", "p1a_seq_free",
+    "p1a_seq_ensure_pages", "p1a_seq_len", "p1a_seq_resident", "p1a_seq_pages", "p1a_seq_host_bytes", "p1a_seq_advance",
+    "p1a_seq_rollback", "p1a_seq_truncate", "p1a_seq_fork", "p1a_seq_offload", "p1a_seq_restore", "p1a_seq_restore_prefix",
+    "p1a_seq_pages_out", "p1a_seq_tokens", "p1a_pool_set_fingerprint", "p1a_pool_fingerprint", "p1a_seq_write", "p1a_seq_read",
+    "p1a_verify_accept",
 ]
 
 
@@ -22,6 +29,15 @@ class p1a_kv(ctypes.Structure):
         ("type", ctypes.c_uint32), ("n_ctx", ctypes.c_int32), ("Hkv", ctypes.c_int32), ("D", ctypes.c_int32),
         ("k", ctypes.c_void_p), ("v", ctypes.c_void_p), ("pt", ctypes.c_void_p), ("rtab", ctypes.c_void_p),
         ("psh", ctypes.c_int32), ("pstride", ctypes.c_size_t),
+    ]
+
+
+class p1a_pool_cfg(ctypes.Structure):
+    _fields_ = [
+        ("kv_type", ctypes.c_uint32), ("n_kv_layers", ctypes.c_int), ("Hkv", ctypes.c_int), ("D", ctypes.c_int),
+        ("psh", ctypes.c_int), ("n_ctx", ctypes.c_int), ("max_slots", ctypes.c_int), ("tokens", ctypes.c_int64),
+        ("reserve_mb", ctypes.c_size_t), ("state_bytes", ctypes.c_size_t), ("host_budget", ctypes.c_size_t),
+        ("host_memory", ctypes.c_int),
     ]
 
 
@@ -74,6 +90,54 @@ def lib():
     L.p1a_release.restype = None
     L.p1a_last_error.restype = ctypes.c_char_p
     L.p1a_version.restype = ctypes.c_char_p
+    # pool / sequence manager (include/p1a_pool.h)
+    pp, ip = ctypes.c_void_p, ctypes.POINTER(ctypes.c_int32)
+    L.p1a_pool_create.restype = pp
+    L.p1a_pool_create.argtypes = [ctypes.POINTER(p1a_pool_cfg), vp]
+    L.p1a_pool_destroy.restype = None
+    L.p1a_pool_destroy.argtypes = [pp]
+    for name in ("p1a_pool_n_pages", "p1a_pool_free_pages", "p1a_pool_max_pages"):
+        getattr(L, name).restype = i32
+        getattr(L, name).argtypes = [pp]
+    for name in ("p1a_pool_page_bytes", "p1a_pool_host_used"):
+        getattr(L, name).restype = sz
+        getattr(L, name).argtypes = [pp]
+    L.p1a_pool_kv_seq.restype = i32
+    L.p1a_pool_kv_seq.argtypes = [pp, i32, i32, kvp]
+    L.p1a_pool_kv_rows.restype = i32
+    L.p1a_pool_kv_rows.argtypes = [pp, i32, kvp]
+    L.p1a_pool_set_rows.restype = i32
+    L.p1a_pool_set_rows.argtypes = [pp, ip, i32]
+    L.p1a_pool_state.restype = vp
+    L.p1a_pool_state.argtypes = [pp, i32]
+    L.p1a_seq_create.restype = i32
+    L.p1a_seq_create.argtypes = [pp]
+    for name in ("p1a_seq_free", "p1a_seq_len", "p1a_seq_resident", "p1a_seq_pages", "p1a_seq_offload", "p1a_seq_restore"):
+        getattr(L, name).restype = i32
+        getattr(L, name).argtypes = [pp, i32]
+    for name in ("p1a_seq_ensure_pages", "p1a_seq_truncate", "p1a_seq_fork", "p1a_seq_restore_prefix"):
+        getattr(L, name).restype = i32
+        getattr(L, name).argtypes = [pp, i32, i32]
+    L.p1a_seq_host_bytes.restype = sz
+    L.p1a_seq_host_bytes.argtypes = [pp, i32]
+    L.p1a_seq_advance.restype = i32
+    L.p1a_seq_advance.argtypes = [pp, i32, ip, i32]
+    L.p1a_seq_rollback.restype = i32
+    L.p1a_seq_rollback.argtypes = [pp, i32, i32, i32]
+    L.p1a_seq_pages_out.restype = i32
+    L.p1a_seq_pages_out.argtypes = [pp, i32, i32, i32, vp]
+    L.p1a_seq_tokens.restype = i32
+    L.p1a_seq_tokens.argtypes = [pp, i32, ip, i32]
+    L.p1a_pool_set_fingerprint.restype = i32
+    L.p1a_pool_set_fingerprint.argtypes = [pp, ctypes.POINTER(ctypes.c_uint64)]
+    L.p1a_pool_fingerprint.restype = i32
+    L.p1a_pool_fingerprint.argtypes = [pp, ctypes.POINTER(ctypes.c_uint64)]
+    L.p1a_seq_write.restype = i32
+    L.p1a_seq_write.argtypes = [pp, i32, ctypes.c_char_p]
+    L.p1a_seq_read.restype = i32
+    L.p1a_seq_read.argtypes = [pp, ctypes.c_char_p]
+    L.p1a_verify_accept.restype = i32
+    L.p1a_verify_accept.argtypes = [ip, ip, i32, i32, ip, ip]
     _lib = L
     return L
 
@@ -231,3 +295,147 @@ def set_nsplit(n):
 
 def bench_skip_merge(on):
     lib().p1a_bench_skip_merge(1 if on else 0)
+
+
+class Pool:
+    """The paged KV pool + sequence manager of include/p1a_pool.h (the reference's tp_model pool / seq_* members).
+
+    Methods keep the reference's names; a refusal raises P1AError with the reference's message. host_memory=True keeps
+    the pool in host memory (no GPU call): `memory()` then returns a numpy view of it."""
+
+    def __init__(self, kv_type, n_kv_layers, Hkv, D, psh, n_ctx, max_slots, tokens, state_bytes=0, host_budget=0,
+                 reserve_mb=0, host_memory=False, stream=None):
+        cfg = p1a_pool_cfg(kv_type, n_kv_layers, Hkv, D, psh, n_ctx, max_slots, tokens, reserve_mb, state_bytes, host_budget,
+                           1 if host_memory else 0)
+        self.cfg, self.host_memory = cfg, host_memory
+        self._p = lib().p1a_pool_create(ctypes.byref(cfg), stream)
+        if not self._p:
+            raise P1AError("alloc_pool refused: " + lib().p1a_last_error().decode())
+
+    def close(self):
+        if self._p:
+            lib().p1a_pool_destroy(self._p)
+            self._p = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def _rc(self, rc, what):
+        if rc < 0:
+            raise P1AError(f"{what} refused (rc={rc}): {lib().p1a_last_error().decode()}")
+        return rc
+
+    n_pages = property(lambda self: lib().p1a_pool_n_pages(self._p))
+    free_pages = property(lambda self: lib().p1a_pool_free_pages(self._p))
+    max_pages = property(lambda self: lib().p1a_pool_max_pages(self._p))
+    page_bytes = property(lambda self: int(lib().p1a_pool_page_bytes(self._p)))
+    host_used = property(lambda self: int(lib().p1a_pool_host_used(self._p)))
+
+    def kv_seq(self, layer, seq):
+        c = p1a_kv()
+        self._rc(lib().p1a_pool_kv_seq(self._p, layer, seq, ctypes.byref(c)), "kv_seq")
+        return c
+
+    def kv_rows(self, layer):
+        c = p1a_kv()
+        self._rc(lib().p1a_pool_kv_rows(self._p, layer, ctypes.byref(c)), "kv_rows")
+        return c
+
+    def set_rows(self, ids):
+        a = (ctypes.c_int32 * len(ids))(*ids)
+        self._rc(lib().p1a_pool_set_rows(self._p, a, len(ids)), "set_rows")
+
+    def state(self, seq):
+        return lib().p1a_pool_state(self._p, seq)
+
+    def seq_create(self):
+        return self._rc(lib().p1a_seq_create(self._p), "seq_create")
+
+    def seq_free(self, seq):
+        self._rc(lib().p1a_seq_free(self._p, seq), "seq_free")
+
+    def ensure_pages(self, seq, n):
+        self._rc(lib().p1a_seq_ensure_pages(self._p, seq, n), "ensure_pages")
+
+    def seq_len(self, seq):
+        return self._rc(lib().p1a_seq_len(self._p, seq), "seq_len")
+
+    def seq_resident(self, seq):
+        return bool(lib().p1a_seq_resident(self._p, seq))
+
+    def seq_pages(self, seq):
+        return self._rc(lib().p1a_seq_pages(self._p, seq), "seq_pages")
+
+    def seq_host_bytes(self, seq):
+        return int(lib().p1a_seq_host_bytes(self._p, seq))
+
+    def seq_advance(self, seq, toks=None, T=None):
+        if toks is None:
+            return self._rc(lib().p1a_seq_advance(self._p, seq, None, T), "seq_advance")
+        a = (ctypes.c_int32 * len(toks))(*toks)
+        return self._rc(lib().p1a_seq_advance(self._p, seq, a, len(toks)), "seq_advance")
+
+    def rollback(self, seq, T, n_keep):
+        return self._rc(lib().p1a_seq_rollback(self._p, seq, T, n_keep), "rollback")
+
+    def seq_truncate(self, seq, n):
+        self._rc(lib().p1a_seq_truncate(self._p, seq, n), "seq_truncate")
+
+    def seq_fork(self, src, n):
+        return self._rc(lib().p1a_seq_fork(self._p, src, n), "seq_fork")
+
+    def seq_offload(self, seq):
+        self._rc(lib().p1a_seq_offload(self._p, seq), "seq_offload")
+
+    def seq_restore(self, seq):
+        self._rc(lib().p1a_seq_restore(self._p, seq), "seq_restore")
+
+    def seq_restore_prefix(self, seq, n):
+        self._rc(lib().p1a_seq_restore_prefix(self._p, seq, n), "seq_restore_prefix")
+
+    def pages_out(self, seq, p0, n, dst_ptr):
+        self._rc(lib().p1a_seq_pages_out(self._p, seq, p0, n, dst_ptr), "pages_out")
+
+    def seq_tokens(self, seq):
+        n = self._rc(lib().p1a_seq_tokens(self._p, seq, None, 0), "seq_tokens")
+        a = (ctypes.c_int32 * max(n, 1))()
+        lib().p1a_seq_tokens(self._p, seq, a, n)
+        return list(a[:n])
+
+    def set_fingerprint(self, fp):
+        a = (ctypes.c_uint64 * 15)(*fp)
+        self._rc(lib().p1a_pool_set_fingerprint(self._p, a), "set_fingerprint")
+
+    def fingerprint(self):
+        a = (ctypes.c_uint64 * 15)()
+        self._rc(lib().p1a_pool_fingerprint(self._p, a), "fingerprint")
+        return list(a)
+
+    def seq_write(self, seq, path):
+        self._rc(lib().p1a_seq_write(self._p, seq, os.fsencode(path)), "seq_write")
+
+    def seq_read(self, path):
+        return self._rc(lib().p1a_seq_read(self._p, os.fsencode(path)), "seq_read")
+
+    def memory(self, c=None):
+        """host-memory pools only: the whole pool as a numpy byte array (a view)"""
+        import numpy as np
+        if not self.host_memory:
+            raise P1AError("memory(): not a host-memory pool")
+        c = c or self.kv_rows(0)
+        n = self.n_pages * self.page_bytes
+        return np.ctypeslib.as_array((ctypes.c_uint8 * n).from_address(c.k))
+
+
+def verify_accept(tokens, greedy, budget):
+    """(rows to keep, accepted drafts, next token) of one verify step: include/p1a_pool.h p1a_verify_accept"""
+    T = len(tokens)
+    a, b = (ctypes.c_int32 * T)(*tokens), (ctypes.c_int32 * T)(*greedy)
+    na, nt = ctypes.c_int32(0), ctypes.c_int32(0)
+    q = lib().p1a_verify_accept(a, b, T, budget, ctypes.byref(na), ctypes.byref(nt))
+    if q < 0:
+        raise P1AError("verify_accept refused: " + lib().p1a_last_error().decode())
+    return q, na.value, nt.value

@@ -8,9 +8,11 @@
 #include <cstdlib>
 #include <cstring>
 #include <numeric>
+#include <string>
 #include <vector>
 
 #include "p100e_fast_attn.hpp"
+#include "p100e_kv_pool.hpp"
 
 namespace F = p100e::fast;
 #define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); exit(2); } } while (0)
@@ -171,9 +173,110 @@ static void test_type(uint32_t type, hipStream_t s) {
     CK(hipFree(q)); CK(hipFree(o1)); CK(hipFree(o2)); CK(hipFree(pool)); CK(hipFree(dtab));
 }
 
+// The pool / sequence manager (include/p100e_kv_pool.hpp) under the attention entry points, in the manner of the
+// reference's tests/fast_sessions_test.cu: two sequences grown in turns (interleaved pages), every step appended to the
+// pool's descriptors and to a contiguous cache; then bitwise checks of decode results across fork, offload + restore
+// (onto other pages) and a session file read into a pool of another size.
+static void test_pool(uint32_t type, hipStream_t s) {
+    printf("  pool %s\n", tname(type));
+    const int L = 2, Hq = 8, Hkv = 2, D = 256, PSH = 4, NCTX = 400, il = 1;
+    const float scale = 0.0625f;
+    p100e::kv_pool pool(type, L, Hkv, D, PSH, NCTX, 3, s, 64);
+    pool.alloc_pool(16 * 40);
+    pool.set_fingerprint({1, 2, 3, 4, 5000, 0, 0, 0, 0, 0, 0, 1, 7, 8, 9});
+    const int a = pool.seq_create(), b = pool.seq_create();
+    F::kv_cache ca = F::kv_alloc(type, NCTX, Hkv, D), cb = F::kv_alloc(type, NCTX, Hkv, D);
+    const int steps[] = {37, 1, 20, 64, 3, 51};
+    int na = 0, nb = 0;
+    for (int st = 0; st < 6; ++st) {
+        const int T = steps[st];
+        for (int which = 0; which < 2; ++which) {
+            const int id = which ? b : a;
+            int & n = which ? nb : na;
+            float * k = dev_rand((size_t) T * Hkv * D, 1.0f), * v = dev_rand((size_t) T * Hkv * D, 1.0f);
+            pool.advance(id, std::vector<int32_t>(T, 100 + st));
+            for (int l = 0; l < L; ++l) { F::kv_cache pc = pool.kv_seq(l, id); F::kv_append(pc, l == il ? k : v, l == il ? v : k, n, T, s); }
+            F::kv_append(which ? cb : ca, k, v, n, T, s);
+            CK(hipStreamSynchronize(s));
+            CK(hipFree(k)); CK(hipFree(v));
+            n += T;
+        }
+    }
+    float * q = dev_rand((size_t) 4 * Hq * D, 0.3f);
+    float * o1, * o2;
+    CK(hipMalloc(&o1, (size_t) 4 * Hq * D * 4)); CK(hipMalloc(&o2, (size_t) 4 * Hq * D * 4));
+    auto dec = [&](const F::kv_cache & c, float * o, int T, int p0) {
+        const bool ok = F::attn_decode(q, c, o, T, p0, Hq, scale, s);
+        CK(hipStreamSynchronize(s));
+        return ok;
+    };
+    auto same = [&](int T) { auto x = bytes_of(o1, (size_t) T * Hq * D * 4), y = bytes_of(o2, (size_t) T * Hq * D * 4); return !memcmp(x.data(), y.data(), x.size()); };
+    bool ok = dec(ca, o1, 4, na - 4) && dec(pool.kv_seq(il, a), o2, 4, na - 4);
+    check("pool descriptors: decode == contiguous cache (interleaved pages)", ok && same(4));
+    ok = dec(cb, o1, 1, nb - 1) && dec(pool.kv_seq(il, b), o2, 1, nb - 1);
+    check("second sequence", ok && same(1));
+    {   // rows of both sequences in one call through the row table
+        pool.set_rows({b, a, a});
+        int32_t hp[3] = {nb - 1, na - 2, na - 1}, * dpos;
+        CK(hipMalloc(&dpos, 12)); CK(hipMemcpy(dpos, hp, 12, hipMemcpyHostToDevice));
+        ok = F::attn_decode_rows(q, pool.kv_rows(il), o2, 3, dpos, Hq, scale, s);
+        CK(hipStreamSynchronize(s));
+        auto rows = bytes_of(o2, (size_t) 3 * Hq * D * 4);
+        const size_t rb = (size_t) Hq * D * 4;
+        const F::kv_cache * cc[3] = {&cb, &ca, &ca};
+        for (int t = 0; t < 3 && ok; ++t) {
+            float * qt = q + (size_t) t * Hq * D;
+            ok = F::attn_decode(qt, *cc[t], o1, 1, hp[t], Hq, scale, s);
+            CK(hipStreamSynchronize(s));
+            auto one = bytes_of(o1, rb);
+            ok = ok && !memcmp(one.data(), rows.data() + t * rb, rb);
+        }
+        check("kv_rows + set_rows: batched rows == one call per row", ok);
+        CK(hipFree(dpos));
+    }
+    const int nf = 100;
+    const int f = pool.seq_fork(a, nf);
+    ok = dec(ca, o1, 1, nf - 1) && dec(pool.kv_seq(il, f), o2, 1, nf - 1);
+    check("seq_fork: the copy decodes like the source", ok && same(1) && pool.seq_len(f) == nf);
+    ok = dec(ca, o1, 4, na - 4);
+    pool.seq_free(f);
+    pool.seq_offload(a);
+    const int filler = pool.seq_create();
+    pool.ensure_pages(filler, 16 * 5);            // the restored sequence lands on other pages
+    pool.seq_restore(a);
+    ok = ok && dec(pool.kv_seq(il, a), o2, 4, na - 4);
+    check("seq_offload + seq_restore onto other pages", ok && same(4) && pool.host_used() == 0);
+    {
+        const std::string path = "/tmp/p1a_mirror_check.p100esq";
+        pool.seq_write(a, path);
+        p100e::kv_pool pool2(type, L, Hkv, D, PSH, 1000, 2, s, 64);
+        pool2.alloc_pool(16 * 64);
+        pool2.set_fingerprint({1, 2, 3, 4, 5000, 0, 0, 0, 0, 0, 0, 1, 7, 8, 9});
+        const int x = pool2.seq_create();
+        pool2.ensure_pages(x, 50);
+        const int r = pool2.seq_read(path);
+        pool2.seq_restore(r);
+        ok = dec(ca, o1, 4, na - 4) && dec(pool2.kv_seq(il, r), o2, 4, na - 4);
+        check("seq_write -> seq_read into a pool of another size", ok && same(4) && pool2.seq_len(r) == na);
+        bool refused = false;
+        p100e::kv_pool pool3(type, L, Hkv, D, PSH + 1, 1000, 2, s, 64);
+        pool3.alloc_pool(32 * 8);
+        pool3.set_fingerprint({1, 2, 3, 4, 5000, 0, 0, 0, 0, 0, 0, 1, 7, 8, 9});
+        try { pool3.seq_read(path); } catch (const std::runtime_error & e) { refused = strstr(e.what(), "page shift") != nullptr; }
+        check("a file of another page size is refused by name", refused);
+        remove(path.c_str());
+    }
+    bool threw = false;
+    try { pool.ensure_pages(a, NCTX + 1); } catch (const std::runtime_error & e) { threw = !strcmp(e.what(), "context full"); }
+    check("refusals throw the engine's messages", threw);
+    F::kv_free(ca); F::kv_free(cb);
+    CK(hipFree(q)); CK(hipFree(o1)); CK(hipFree(o2));
+}
+
 int main() {
     hipStream_t s; CK(hipStreamCreate(&s));
     for (uint32_t type : {F::KV_F16, F::KV_Q8_0, F::KV_Q4_0}) test_type(type, s);
+    for (uint32_t type : {F::KV_F16, F::KV_Q8_0, F::KV_Q4_0}) test_pool(type, s);
     p1a_release();
     printf("%d checks, %d failed\n", g_checks, g_fail);
     return g_fail ? 1 : 0;
