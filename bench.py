@@ -146,6 +146,7 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
     ex["verify_4x4_q4_0_64K_us"] = round(sec * 1e6, 2)
     ex["verify_GBs"] = round(vb / sec / 1e9, 1)
     del kv, cr
+    ex.update(mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale))
     # configs[2]: 8 slots, one row each, ctx log-uniform in [1024, 32768], q8_0, one shared pool
     rs = torch.Generator().manual_seed(8)
     lens = [int(math.exp(float(torch.empty(1).uniform_(math.log(1024), math.log(32768), generator=rs)))) for _ in range(8)]
@@ -163,6 +164,73 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
     ex["batched_GBs"] = round(bb / sec / 1e9, 1)
     ex["batched_ctx"] = lens
     return ex
+
+
+def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, steps=30):
+    """The verify attention inside a step loop, as the engine's scheduler drives it (accept / rollback per sequence,
+    src/sched.cpp:1053-1087 of the reference): 4 sequences of a q4_0 pool at ~64K tokens, every step 1 + 3 draft rows per
+    sequence go through attn_prep (norm, rope, quantizing KV write at each row's own position) and one batched
+    attn_decode_rows, the host accepts a prefix (each draft right with probability 0.7, seeded) and rolls the rest back.
+    Wall time per step, host bookkeeping and the position upload included."""
+    import random
+    import time
+    pool = p1a.Pool(p1a.KV_Q4_0, 1, Hkv, D, psh, n_ctx=ctx + 4096, max_slots=n_seq, tokens=n_seq * (ctx + 4096))
+    g = torch.Generator(device="cuda").manual_seed(31)
+    ids = [pool.seq_create() for _ in range(n_seq)]
+    for i, s in enumerate(ids):
+        n = ctx - 37 * i                                    # unequal depths
+        for a in range(0, n, 8192):
+            T = min(8192, n - a)
+            k = torch.randn((T, Hkv, D), generator=g, device="cuda")
+            k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + 1e-6)
+            v = torch.randn((T, Hkv, D), generator=g, device="cuda")
+            pool.seq_advance(s, T=T)
+            p1a.kv_append(pool.cache_seq(0, s), k, v, a, T)
+    torch.cuda.synchronize()
+    R = 4
+    rows = n_seq * R
+    qg = torch.randn((rows, Hq, 2 * D), generator=g, device="cuda")
+    kx = torch.randn((rows, Hkv, D), generator=g, device="cuda")
+    vx = torch.randn((rows, Hkv, D), generator=g, device="cuda")
+    w = torch.ones(D, device="cuda")
+    q = torch.empty((rows, Hq, D), device="cuda")
+    gate = torch.empty((rows, Hq * D), device="cuda")
+    out = torch.empty((rows, Hq, D), device="cuda")
+    pos_h = torch.empty(rows, dtype=torch.int32).pin_memory()
+    pos = torch.empty(rows, dtype=torch.int32, device="cuda")
+    pool.set_rows([s for s in ids for _ in range(R)])
+    cr = pool.cache_rows(0)
+    rnd = random.Random(7)
+    emitted, t_total = 0, 0.0
+    for step in range(steps + 3):
+        t0 = time.perf_counter()
+        for i, s in enumerate(ids):
+            n = pool.seq_len(s)
+            for t in range(R):
+                pos_h[i * R + t] = n + t
+            pool.seq_advance(s, T=R)
+        pos.copy_(pos_h, non_blocking=True)
+        p1a.attn_prep(qg, kx, vx, w, w, pos, q, gate, cr, -1, rows, Hq, 64, 1e7, 1e-6)
+        p1a.attn_decode_rows(q, cr, out, rows, pos, Hq, scale, gate=gate, rows_per_seq=R)
+        torch.cuda.synchronize()                            # the engine reads the rows' logits here
+        n_out = 0
+        for s in ids:
+            tokens = [1, 2, 3, 4]
+            greedy = [2, 3, 4, 5]
+            for d in range(R - 1):
+                if rnd.random() > 0.7:
+                    greedy[d] = 0                           # draft d + 1 was wrong
+                    break
+            keep, _, _ = p1a.verify_accept(tokens, greedy, 1 << 20)
+            pool.rollback(s, R, keep)
+            n_out += keep
+        dt = time.perf_counter() - t0
+        if step >= 3:
+            t_total += dt
+            emitted += n_out
+    pool.close()
+    return {"mtp_verify_step_us": round(t_total / steps * 1e6, 1), "mtp_tokens_per_step": round(emitted / steps, 2),
+            "mtp_loop": f"{n_seq} sequences x (1 + 3 drafts), q4_0, ~{ctx} tokens each, prep + decode + accept/rollback, wall clock"}
 
 
 def cpu_baseline(Hq, Hkv, D, n_ctx, seed):

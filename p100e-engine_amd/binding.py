@@ -163,9 +163,10 @@ def _stream():
 class KVCache:
     """Device KV cache of one layer, the twin of the reference's kv_cache (src/fast/attn.cuh:18-32).
 
-    Contiguous: KVCache.contiguous(type, n_ctx, Hkv, D). Paged: KVCache.paged(...) lays a pool out as the engine does
-    (src/tp_model.cu:3880-3942 of the reference): [page][layer][K|V][2^psh positions][row], one layer selected by the
-    k / v base pointers, a slot by its page-table row.
+    Contiguous: KVCache.contiguous(type, n_ctx, Hkv, D). Paged: KVCache.paged(...) lays a test pool out as
+    [page][layer][K|V][2^psh positions][row] - a page stride that spans other layers, as the reference's session test
+    does (tests/fast_sessions_test.cu:75,91-92) - one layer selected by the k / v base pointers, a slot by its
+    page-table row. (The engine's own pool layout is class Pool's.)
     """
 
     def __init__(self, kv_type, n_ctx, Hkv, D, k, v, pt=None, rtab=None, psh=0, pstride=0, keep=()):
@@ -297,6 +298,16 @@ def bench_skip_merge(on):
     lib().p1a_bench_skip_merge(1 if on else 0)
 
 
+class KVDesc:
+    """A p1a_kv descriptor that somebody else owns the memory of (the pool's)."""
+
+    def __init__(self, st):
+        self._st = st
+
+    def struct(self):
+        return self._st
+
+
 class Pool:
     """The paged KV pool + sequence manager of include/p1a_pool.h (the reference's tp_model pool / seq_* members).
 
@@ -333,6 +344,13 @@ class Pool:
     max_pages = property(lambda self: lib().p1a_pool_max_pages(self._p))
     page_bytes = property(lambda self: int(lib().p1a_pool_page_bytes(self._p)))
     host_used = property(lambda self: int(lib().p1a_pool_host_used(self._p)))
+
+    def cache_seq(self, layer, seq):
+        """kv_seq as an object the attention entry points of this module take"""
+        return KVDesc(self.kv_seq(layer, seq))
+
+    def cache_rows(self, layer):
+        return KVDesc(self.kv_rows(layer))
 
     def kv_seq(self, layer, seq):
         c = p1a_kv()
