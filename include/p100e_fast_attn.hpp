@@ -80,13 +80,23 @@ inline bool kv_append_rows(kv_cache & c, const float * k, const float * v, const
     return p1a_kv_append(&p, k, v, -1, nullptr, pos, T, s) == P1A_OK;
 }
 
-// src/fast/fused.cuh:101-113 (Hkv and D must be the cache's; the interleaved M-RoPE argument is not mirrored)
+// src/fast/mrope.cuh:14-19, field for field
+struct mrope_pos {
+    const int32_t * p = nullptr;   // device [3][stride] positions (t, h, w) of the rows; nullptr = plain NEOX
+    int stride = 0;                // row stride between the three streams
+    int s0 = 0, s1 = 0, s2 = 0;    // sections (in rotary pairs)
+    int sect = 0;                  // sum of all sections
+};
+
+// src/fast/fused.cuh:101-113 (Hkv and D must be the cache's)
 inline bool attn_prep(const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
                       const int32_t * pos, float * q, float * gate, kv_cache & c, int p0, int T, int Hq, int Hkv, int D,
-                      int n_rot, float freq_base, float eps, hipStream_t s, int ldq = 0, int ldk = 0, int ldv = 0) {
+                      int n_rot, float freq_base, float eps, hipStream_t s, int ldq = 0, int ldk = 0, int ldv = 0,
+                      const mrope_pos & mr = mrope_pos{}) {
     if (Hkv != c.Hkv || D != c.D) return false;
     const p1a_kv p = detail::pod(c);
-    return p1a_attn_prep(qg, k, v, q_norm, k_norm, pos, q, gate, &p, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, s) == P1A_OK;
+    return p1a_attn_prep_mrope(qg, k, v, q_norm, k_norm, pos, q, gate, &p, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv,
+                               mr.p, mr.stride, mr.s0, mr.s1, mr.s2, mr.sect, s) == P1A_OK;
 }
 
 // src/fast/fused.cuh:91-98

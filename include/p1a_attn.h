@@ -87,13 +87,24 @@ int p1a_kv_append(const p1a_kv *c, const float *k, const float *v, int p0, const
  * with rmsnorm(x) = x / sqrt(mean(x^2) + eps) per head, the NEOX rotation of dims (j, j + n_rot/2), j < n_rot/2, by
  * pos[t] * freq_base^(-2j/n_rot), and the quantizing write of p1a_kv_append. The cache row of token t is p0 + t, or
  * pos[t] (read on the device, own page table pt + rtab[t]) when p0 < 0; the rotary position is pos[t] in both cases.
- * ld* = 0 means dense rows; q_norm / k_norm ([D]) may be NULL. D <= 256, n_rot % 8 == 0; interleaved M-RoPE is not covered.
+ * ld* = 0 means dense rows; q_norm / k_norm ([D]) may be NULL. D <= 256, n_rot % 8 == 0.
  * Replaces the front half of attn_prep (src/fast/fused.cuh:101-113, kernel src/fast/fused.cu:512-573) = k::split_q_gate
  * + fast::rmsnorm + k::rope_neox + kv_append of the unfused path (src/tp_model.cu:1717-1734).
  */
 int p1a_attn_prep(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
                   const int32_t *pos, float *q, float *gate, const p1a_kv *c, int p0, int T, int Hq, int n_rot,
                   float freq_base, float eps, int ldq, int ldk, int ldv, void *stream);
+/*
+ * The same with interleaved M-RoPE positions (images in the context): mr_pos [3][mr_stride] holds the t / h / w positions
+ * of the rows; rotary pair j takes the stream its sector = j % sect selects (sector % 3 == 1 and < 3 s1 -> h,
+ * % 3 == 2 and < 3 s2 -> w, % 3 == 0 and < 3 s0 -> t, otherwise position 0); s0, s1, s2 are the sections in rotary
+ * pairs, sect the sum of all four. Cache rows still come from pos / p0. mr_pos == NULL is p1a_attn_prep.
+ * Replaces attn_prep with mr.p != nullptr (src/fast/fused.cuh:108-113, src/fast/mrope.cuh:14-33).
+ */
+int p1a_attn_prep_mrope(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
+                        const int32_t *pos, float *q, float *gate, const p1a_kv *c, int p0, int T, int Hq, int n_rot,
+                        float freq_base, float eps, int ldq, int ldk, int ldv, const int32_t *mr_pos, int mr_stride,
+                        int s0, int s1, int s2, int sect, void *stream);
 
 /*
  * Decode / MTP-verify attention: q, out [T][Hq][D] f32;

@@ -200,7 +200,21 @@ void orc_rmsnorm_heads(float *x, size_t nheads, int D, float eps) {
  * rotation angle is pos * (float) pow(base, -2j/n_rot) in fp32 and its cosine / sine are the double-precision ones
  * rounded to fp32; products and sums are rounded separately (no fused multiply-add).
  */
-static void prep_norm_rope(const float *src, const float *w, int D, int n_rot, float freq_base, float eps, int pos, float *dst) {
+/* interleaved M-RoPE (src/fast/mrope.cuh:1-8, 25-33): rotary pair j takes the position of one of three streams by its
+ * sector = j % sect: sector % 3 == 1 and < 3 s1 -> h; sector % 3 == 2 and < 3 s2 -> w; sector % 3 == 0 and < 3 s0 -> t;
+ * anything else -> the 4th stream, which is 0. mr == NULL: every pair takes pos. */
+static int mrope_pick(const orc_mrope *mr, int t, int j, int pos) {
+    if (!mr || !mr->p) return pos;
+    const int sector = j % mr->sect;
+    int s;
+    if (sector % 3 == 1 && sector < 3 * mr->s1) s = 1;
+    else if (sector % 3 == 2 && sector < 3 * mr->s2) s = 2;
+    else if (sector % 3 == 0 && sector < 3 * mr->s0) s = 0;
+    else return 0;
+    return mr->p[(size_t) s * mr->stride + t];
+}
+
+static void prep_norm_rope(const float *src, const float *w, int D, int n_rot, float freq_base, float eps, int pos, const orc_mrope *mr, int t, float *dst) {
     float part[64];
     for (int i = 0; i < 64; ++i) {
         part[i] = 0.0f;
@@ -224,7 +238,7 @@ static void prep_norm_rope(const float *src, const float *w, int D, int n_rot, f
     const int half = n_rot / 2;
     for (int j = 0; j < half; ++j) {
         const float inv = (float) pow((double) freq_base, -2.0 * (double) j / (double) n_rot);
-        const float theta = (float) pos * inv;
+        const float theta = (float) mrope_pick(mr, t, j, pos) * inv;
         const float c = (float) cos((double) theta), sn = (float) sin((double) theta);
         const float x0 = dst[j], x1 = dst[j + half];
         const float a0 = x0 * c, a1 = x1 * sn, b0 = x0 * sn, b1 = x1 * c;
@@ -236,6 +250,13 @@ static void prep_norm_rope(const float *src, const float *w, int D, int n_rot, f
 int orc_attn_prep(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
                   const int32_t *pos, float *q, float *gate, const orc_kv *c, int p0, int T, int Hq, int Hkv, int D,
                   int n_rot, float freq_base, float eps, int ldq, int ldk, int ldv) {
+    return orc_attn_prep_mrope(qg, k, v, q_norm, k_norm, pos, q, gate, c, p0, T, Hq, Hkv, D, n_rot, freq_base, eps, ldq, ldk, ldv, NULL);
+}
+
+int orc_attn_prep_mrope(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
+                        const int32_t *pos, float *q, float *gate, const orc_kv *c, int p0, int T, int Hq, int Hkv, int D,
+                        int n_rot, float freq_base, float eps, int ldq, int ldk, int ldv, const orc_mrope *mr) {
+    if (mr && mr->p && mr->sect <= 0) return -1;
     if (!pos || D % 32 || D > 256 || n_rot % 8 || n_rot > D || c->D != D || c->Hkv != Hkv) return -1;
     if (!ldq) ldq = Hq * 2 * D;
     if (!ldk) ldk = Hkv * D;
@@ -247,10 +268,10 @@ int orc_attn_prep(const float *qg, const float *k, const float *v, const float *
         for (int h = 0; h < Hq; ++h) {
             const float *src = qg + (size_t) t * ldq + (size_t) h * 2 * D;
             memcpy(gate + ((size_t) t * Hq + h) * D, src + D, sizeof(float) * D);
-            prep_norm_rope(src, q_norm, D, n_rot, freq_base, eps, pos[t], q + ((size_t) t * Hq + h) * D);
+            prep_norm_rope(src, q_norm, D, n_rot, freq_base, eps, pos[t], mr, t, q + ((size_t) t * Hq + h) * D);
         }
         for (int h = 0; h < Hkv; ++h) {
-            prep_norm_rope(k + (size_t) t * ldk + (size_t) h * D, k_norm, D, n_rot, freq_base, eps, pos[t], kr + (size_t) h * D);
+            prep_norm_rope(k + (size_t) t * ldk + (size_t) h * D, k_norm, D, n_rot, freq_base, eps, pos[t], mr, t, kr + (size_t) h * D);
             memcpy(vr + (size_t) h * D, v + (size_t) t * ldv + (size_t) h * D, sizeof(float) * D);
         }
         /* row t of the batch: its own page table (rtab[t]) and its own position */

@@ -17,6 +17,9 @@
  *   orc_attn_prep                              : numpy float64 restatement of norm * weight and the NEOX rotation (to a few
  *       fp32 ulps); closed forms (position 0 rotates nothing, the rotation keeps pair norms, q . k after rope depends on
  *       the position difference only, a constant head norms to w); KV rows == orc_kv_append_rows of the normed, roped k.
+ *   orc_attn_prep_mrope                        : t = h = w = p is bitwise plain NEOX at p (src/fast/mrope.cuh:6-7); the
+ *       stream of every rotary pair from a table written out by hand from the rule's words for sections [11, 11, 10, 0]
+ *       and [2, 1, 1, 0]; moving one stream changes exactly the pairs of that stream.
  *   orc_a16_quant                              : an independent numpy float32 restatement (element -> slot map written out
  *       from the engine's comment, not from its index arithmetic), closed forms (zero group, unit group, clamp at 65520).
  * No function of this file is "parity unpinned".
@@ -72,6 +75,18 @@ void orc_rmsnorm_heads(float *x, size_t nheads, int D, float eps);
 int orc_attn_prep(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
                   const int32_t *pos, float *q, float *gate, const orc_kv *c, int p0, int T, int Hq, int Hkv, int D,
                   int n_rot, float freq_base, float eps, int ldq, int ldk, int ldv);
+/* the same with interleaved M-RoPE positions (src/fast/mrope.cuh:14-33, src/fast/fused.cuh:108-113): rotary pair j of
+ * row t rotates by the position of the stream its sector selects; cache rows still come from pos / p0. mr == NULL or
+ * mr->p == NULL: plain NEOX. */
+typedef struct orc_mrope {
+    const int32_t *p;   /* [3][stride]: t, h, w positions of the rows */
+    int stride;
+    int s0, s1, s2;     /* sections, in rotary pairs */
+    int sect;           /* sum of all four sections */
+} orc_mrope;
+int orc_attn_prep_mrope(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
+                        const int32_t *pos, float *q, float *gate, const orc_kv *c, int p0, int T, int Hq, int Hkv, int D,
+                        int n_rot, float freq_base, float eps, int ldq, int ldk, int ldv, const orc_mrope *mr);
 /* a16 activation quantize (src/fast/a16q.cuh:21-45 = src/fast/matvec_a16.cu:29-100): y [T][n] f32, n % 32 == 0 ->
  * qbuf: T * n/32 * 16 half2 of scaled values (slot order of the engine), then T * n/32 half2 (amax, sum). */
 void orc_a16_quant(const float *y, int T, int n, uint16_t *qbuf);

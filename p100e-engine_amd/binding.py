@@ -7,7 +7,7 @@ import os
 KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
-    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
+    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_release", "p1a_last_error",
     "p1a_version",
     # include/p1a_pool.h
@@ -65,6 +65,8 @@ def lib():
     L.p1a_kv_append.argtypes = [kvp, vp, vp, i32, vp, vp, i32, vp]
     L.p1a_attn_prep.restype = i32
     L.p1a_attn_prep.argtypes = [vp] * 8 + [kvp, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp]
+    L.p1a_attn_prep_mrope.restype = i32
+    L.p1a_attn_prep_mrope.argtypes = [vp] * 8 + [kvp, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp, i32, i32, i32, i32, i32, vp]
     L.p1a_attn_decode_a16.restype = i32
     L.p1a_attn_decode_a16.argtypes = [vp, kvp, vp, vp, vp, i32, i32, vp, vp, i32, i32, f32, vp]
     L.p1a_a16_bytes.restype = sz
@@ -236,9 +238,16 @@ def kv_append_rows(c, k, v, pos_rows, T):
     _check(lib().p1a_kv_append(ctypes.byref(c.struct()), _ptr(k), _ptr(v), -1, None, _ptr(pos_rows), T, _stream()), "kv_append_rows")
 
 
-def attn_prep(qg, k, v, q_norm, k_norm, pos, q, gate, c, p0, T, Hq, n_rot, freq_base, eps, ldq=0, ldk=0, ldv=0):
+def attn_prep(qg, k, v, q_norm, k_norm, pos, q, gate, c, p0, T, Hq, n_rot, freq_base, eps, ldq=0, ldk=0, ldv=0, mrope=None):
     """src/fast/fused.cuh:101-113: q | gate split, per-head RMS norm * weight, NEOX rope, quantizing KV write (p0 < 0:
-    cache row of token t = pos[t], its own page table)."""
+    cache row of token t = pos[t], its own page table). mrope = (positions int32 [3][stride] on the device, stride,
+    (s0, s1, s2), sect): interleaved M-RoPE (src/fast/mrope.cuh)."""
+    if mrope is not None:
+        mp, stride, (s0, s1, s2), sect = mrope
+        _check(lib().p1a_attn_prep_mrope(_ptr(qg), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(pos), _ptr(q), _ptr(gate),
+                                         ctypes.byref(c.struct()), p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv,
+                                         _ptr(mp), stride, s0, s1, s2, sect, _stream()), "attn_prep")
+        return
     _check(lib().p1a_attn_prep(_ptr(qg), _ptr(k), _ptr(v), _ptr(q_norm), _ptr(k_norm), _ptr(pos), _ptr(q), _ptr(gate),
                                ctypes.byref(c.struct()), p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, _stream()), "attn_prep")
 

@@ -110,7 +110,19 @@ int p1a_kv_append(const p1a_kv * c, const float * k, const float * v, int p0, co
 int p1a_attn_prep(const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
                   const int32_t * pos, float * q, float * gate, const p1a_kv * c, int p0, int T, int Hq, int n_rot,
                   float freq_base, float eps, int ldq, int ldk, int ldv, void * stream) {
+    return p1a_attn_prep_mrope(qg, k, v, q_norm, k_norm, pos, q, gate, c, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv,
+                               nullptr, 0, 0, 0, 0, 0, stream);
+}
+
+int p1a_attn_prep_mrope(const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
+                        const int32_t * pos, float * q, float * gate, const p1a_kv * c, int p0, int T, int Hq, int n_rot,
+                        float freq_base, float eps, int ldq, int ldk, int ldv, const int32_t * mr_pos, int mr_stride,
+                        int s0, int s1, int s2, int sect, void * stream) {
     if (!kv_ok(c, "p1a_attn_prep")) return P1A_E_ARG;
+    if (mr_pos && (sect <= 0 || mr_stride < T || s0 < 0 || s1 < 0 || s2 < 0)) {
+        set_error("p1a_attn_prep: M-RoPE needs sect > 0, sections >= 0 and a stream stride of at least T (sect=%d stride=%d)", sect, mr_stride);
+        return P1A_E_ARG;
+    }
     if (!qg || !k || !v || !pos || !q || !gate || T < 0 || Hq < 1) { set_error("p1a_attn_prep: null argument or bad T / Hq"); return P1A_E_ARG; }
     if (T == 0) return P1A_OK;
     const int D = c->D, Hkv = c->Hkv;
@@ -126,7 +138,8 @@ int p1a_attn_prep(const float * qg, const float * k, const float * v, const floa
         set_error("p1a_attn_prep: pointers must be 16-byte aligned, row strides multiples of 4 floats and at least one row");
         return P1A_E_SHAPE;
     }
-    return launch_prep(*c, qg, k, v, q_norm, k_norm, pos, q, gate, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, (hipStream_t) stream);
+    const mrope_view mr{mr_pos, mr_stride, s0, s1, s2, sect};
+    return launch_prep(*c, qg, k, v, q_norm, k_norm, pos, q, gate, p0, T, Hq, n_rot, freq_base, eps, ldq, ldk, ldv, mr, (hipStream_t) stream);
 }
 
 size_t p1a_a16_bytes(int T, int n) { return T < 0 || n < 0 ? 0 : (size_t) T * (size_t) (n / 32) * 17 * 4; }

@@ -123,7 +123,7 @@ __global__ void __launch_bounds__(64) prep_k(const float * __restrict__ qg, cons
                                              const float * __restrict__ kn, const int32_t * __restrict__ pos,
                                              float * __restrict__ q, float * __restrict__ gate, char * kc, char * vc, int p0,
                                              int Hq, int Hkv, int D, int n_rot, float freq_base, float eps, int ldq, int ldk,
-                                             int ldv, kv_view pg) {
+                                             int ldv, kv_view pg, mrope_view mr) {
     const int t = blockIdx.y, b = blockIdx.x, i = threadIdx.x;
     const bool live = 4 * i < D;                               // dead lanes form whole 8-lane groups (D % 32 == 0)
     const int row = p0 < 0 ? pos[t] : p0 + t;                  // cache position of token t (src/fast/fused.cu:520)
@@ -171,7 +171,17 @@ __global__ void __launch_bounds__(64) prep_k(const float * __restrict__ qg, cons
     const int half = n_rot >> 1, hl = half >> 2;
     const bool lo = i < hl, rot = i < 2 * hl;
     const int partner = lo ? i + hl : i - hl;
-    const float posf = (float) pos[t];
+    // interleaved M-RoPE (src/fast/mrope.cuh:25-33): pair j rotates by the position of the stream its sector selects
+    auto pair_pos = [&](int j) {
+        if (!mr.p) return pos[t];
+        const int sector = j % mr.sect;
+        int st;
+        if (sector % 3 == 1 && sector < 3 * mr.s1) st = 1;
+        else if (sector % 3 == 2 && sector < 3 * mr.s2) st = 2;
+        else if (sector % 3 == 0 && sector < 3 * mr.s0) st = 0;
+        else return 0;
+        return mr.p[(size_t) st * mr.stride + t];
+    };
     // the angle tables of the head: pair j is computed once, by lane j & 63 (slot j >> 6), and handed round by shuffle
     float tc[2] = {1.f, 1.f}, tsn[2] = {0.f, 0.f};
 #pragma unroll
@@ -179,7 +189,7 @@ __global__ void __launch_bounds__(64) prep_k(const float * __restrict__ qg, cons
         const int jj = i + 64 * sl;
         if (jj < half) {
             const float inv = (float) pow((double) freq_base, -2.0 * (double) jj / (double) n_rot);
-            const float theta = posf * inv;
+            const float theta = (float) pair_pos(jj) * inv;
             tc[sl] = (float) cos((double) theta);
             tsn[sl] = (float) sin((double) theta);
         }
@@ -247,12 +257,12 @@ int launch_ew_quant(int op, const float * a, const float * b, float * y, void * 
 
 int launch_prep(const p1a_kv & c, const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
                 const int32_t * pos, float * q, float * gate, int p0, int T, int Hq, int n_rot, float freq_base, float eps,
-                int ldq, int ldk, int ldv, hipStream_t s) {
+                int ldq, int ldk, int ldv, const mrope_view & mr, hipStream_t s) {
     const kv_view pg = view_of(c);
     const dim3 grid(Hq + 2 * c.Hkv, T);
     char * kc = (char *) c.k, * vc = (char *) c.v;
 #define P1A_PREP(KT_) prep_k<KT_><<<grid, 64, 0, s>>>(qg, k, v, q_norm, k_norm, pos, q, gate, kc, vc, p0, Hq, c.Hkv, c.D, n_rot, \
-                                                      freq_base, eps, ldq, ldk, ldv, pg)
+                                                      freq_base, eps, ldq, ldk, ldv, pg, mr)
     if (c.type == P1A_KV_F16) P1A_PREP(P1A_KV_F16);
     else if (c.type == P1A_KV_Q8_0) P1A_PREP(P1A_KV_Q8_0);
     else P1A_PREP(P1A_KV_Q4_0);

@@ -101,9 +101,11 @@ int decode_rows_per_group(const p1a_kv & c, int Hq, int want);
 int decode_nsplit(const p1a_kv & c, int Hq, int nsplit_req, int cus);
 void decode_scratch_need(const p1a_kv & c, int Hq, int rows, int rows_per_group, int nsplit_req, int cus,
                          size_t & bytes_o, size_t & bytes_ml);
+// interleaved M-RoPE positions of a batch (src/fast/mrope.cuh:14-19): [3][stride] t / h / w, sections in rotary pairs
+struct mrope_view { const int32_t * p; int stride, s0, s1, s2, sect; };
 int launch_prep(const p1a_kv & c, const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
                 const int32_t * pos, float * q, float * gate, int p0, int T, int Hq, int n_rot, float freq_base, float eps,
-                int ldq, int ldk, int ldv, hipStream_t s);
+                int ldq, int ldk, int ldv, const mrope_view & mr, hipStream_t s);
 int launch_ew_quant(int op, const float * a, const float * b, float * y, void * qbuf, int T, int n, int lda, int ldb, hipStream_t s);
 int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s);

@@ -17,6 +17,11 @@ class orc_kv(ctypes.Structure):
     ]
 
 
+class orc_mrope(ctypes.Structure):
+    _fields_ = [("p", ctypes.c_void_p), ("stride", ctypes.c_int), ("s0", ctypes.c_int), ("s1", ctypes.c_int),
+                ("s2", ctypes.c_int), ("sect", ctypes.c_int)]
+
+
 _lib = None
 
 
@@ -46,6 +51,8 @@ def lib():
         L.orc_rmsnorm_heads.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_float]
         L.orc_attn_prep.argtypes = [ctypes.c_void_p] * 8 + [ctypes.POINTER(orc_kv)] + [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_float] + [ctypes.c_int] * 3
         L.orc_attn_prep.restype = ctypes.c_int
+        L.orc_attn_prep_mrope.argtypes = L.orc_attn_prep.argtypes + [ctypes.POINTER(orc_mrope)]
+        L.orc_attn_prep_mrope.restype = ctypes.c_int
         L.orc_a16_quant.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         L.orc_num_threads.restype = ctypes.c_int
         _lib = L
@@ -149,8 +156,9 @@ def rmsnorm_heads(x, D, eps=1e-6):
     return x
 
 
-def attn_prep(c, qg, k, v, q_norm, k_norm, pos, p0, Hq, n_rot, freq_base, eps=1e-6):
-    """q | gate split, norm, rope, quantize-append: returns (q, gate); K / V rows are written into c."""
+def attn_prep(c, qg, k, v, q_norm, k_norm, pos, p0, Hq, n_rot, freq_base, eps=1e-6, mrope=None):
+    """q | gate split, norm, rope, quantize-append: returns (q, gate); K / V rows are written into c.
+    mrope = (positions int32 [3][stride], (s0, s1, s2), sect): interleaved M-RoPE."""
     qg = np.ascontiguousarray(qg, np.float32)
     k = np.ascontiguousarray(k, np.float32)
     v = np.ascontiguousarray(v, np.float32)
@@ -160,8 +168,15 @@ def attn_prep(c, qg, k, v, q_norm, k_norm, pos, p0, Hq, n_rot, freq_base, eps=1e
     gate = np.zeros((T, Hq * c.D), np.float32)
     qn = None if q_norm is None else np.ascontiguousarray(q_norm, np.float32)
     kn = None if k_norm is None else np.ascontiguousarray(k_norm, np.float32)
-    rc = lib().orc_attn_prep(_p(qg), _p(k), _p(v), _p(qn), _p(kn), _p(pos), _p(q), _p(gate), ctypes.byref(c.struct()), p0, T, Hq,
-                             c.Hkv, c.D, n_rot, freq_base, eps, 0, 0, 0)
+    if mrope is None:
+        rc = lib().orc_attn_prep(_p(qg), _p(k), _p(v), _p(qn), _p(kn), _p(pos), _p(q), _p(gate), ctypes.byref(c.struct()), p0, T, Hq,
+                                 c.Hkv, c.D, n_rot, freq_base, eps, 0, 0, 0)
+    else:
+        mp, (s0, s1, s2), sect = mrope
+        mp = np.ascontiguousarray(mp, np.int32)
+        mr = orc_mrope(mp.ctypes.data, mp.shape[1], s0, s1, s2, sect)
+        rc = lib().orc_attn_prep_mrope(_p(qg), _p(k), _p(v), _p(qn), _p(kn), _p(pos), _p(q), _p(gate), ctypes.byref(c.struct()), p0, T,
+                                       Hq, c.Hkv, c.D, n_rot, freq_base, eps, 0, 0, 0, ctypes.byref(mr))
     assert rc == 0, rc
     return q, gate
 

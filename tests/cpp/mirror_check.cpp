@@ -160,6 +160,16 @@ static void test_type(uint32_t type, hipStream_t s) {
             ok = ok && !memcmp(hv.data() + (size_t) p * rowb, hpool.data() + o + PS * rowb, rowb);
         }
         check("attn_prep host positions vs device positions + page table", ok);
+        {   // text rows through the M-RoPE argument (t = h = w = p) give the plain call's bits
+            int32_t * d3; CK(hipMalloc(&d3, 3 * T * 4));
+            for (int i = 0; i < 3; ++i) CK(hipMemcpy(d3 + i * T, hp.data(), T * 4, hipMemcpyHostToDevice));
+            F::mrope_pos mr; mr.p = d3; mr.stride = T; mr.s0 = 11; mr.s1 = 11; mr.s2 = 10; mr.sect = 32;
+            const bool a3 = F::attn_prep(qg, kk, vv, wn, wn, dpos, o2, g2, cc[sq], p0, T, Hq, Hkv, D, n_rot, 1e7f, 1e-6f, s, 0, 0, 0, mr);
+            CK(hipStreamSynchronize(s));
+            auto qc = bytes_of(o2, (size_t) T * Hq * D * 4);
+            check("attn_prep with M-RoPE positions of text rows == plain", a3 && !memcmp(qa.data(), qc.data(), qa.size()));
+            CK(hipFree(d3));
+        }
         CK(hipFree(qg)); CK(hipFree(kk)); CK(hipFree(vv)); CK(hipFree(wn)); CK(hipFree(g1)); CK(hipFree(g2)); CK(hipFree(dpos)); CK(hipFree(drt));
     }
     {   // a refusal launches nothing and leaves out untouched

@@ -166,3 +166,40 @@ def test_decode_emits_a16(p1a, kv_type):
     torch.cuda.synchronize()
     assert torch.equal(o1, o2)
     assert np.array_equal(qb.cpu().numpy().view(np.uint16), O.a16_quant(o2.cpu().numpy().reshape(T, Hq * D)))
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_mrope_positions(p1a, kv_type):
+    """interleaved M-RoPE (src/fast/mrope.cuh): image rows with their own t / h / w, the same bars as the plain rotation;
+    and text rows (t = h = w = p) give the plain call's bits."""
+    Hq, Hkv, D, n_rot, T, n_ctx, base, eps = 24, 4, 256, 64, 9, 64, 1e7, 1e-6
+    qg, k, v, qn, kn = make(77, T, Hq, Hkv, D)
+    pos = (20 + np.arange(T)).astype(np.int32)                            # cache rows
+    P = 1000                                                               # a 3 x 3 image placed at P: t = P, h = P + i / 3, w = P + i % 3
+    mp = np.zeros((3, T + 3), np.int32)                                   # (a stride larger than T)
+    mp[0, :T], mp[1, :T], mp[2, :T] = P, P + np.arange(T) // 3, P + np.arange(T) % 3
+    host = O.HostKV.contiguous(kv_type, n_ctx, Hkv, D)
+    q_ref, gate_ref = O.attn_prep(host, qg, k, v, qn, kn, pos, -1, Hq, n_rot, base, eps, mrope=(mp, (11, 11, 10), 32))
+    c = p1a.KVCache.contiguous(kv_type, n_ctx, Hkv, D)
+    q = torch.zeros((T, Hq, D), device="cuda")
+    gate = torch.zeros((T, Hq * D), device="cuda")
+    p1a.attn_prep(dev(qg), dev(k), dev(v), dev(qn), dev(kn), dev(pos), q, gate, c, -1, T, Hq, n_rot, base, eps,
+                  mrope=(dev(mp), T + 3, (11, 11, 10), 32))
+    torch.cuda.synchronize()
+    assert np.array_equal(gate.cpu().numpy(), gate_ref)
+    qd = q.cpu().numpy()
+    assert ulp_diff(qd, q_ref).max() <= 1 and np.mean(qd.view(np.int32) == q_ref.view(np.int32)) > 0.999
+    assert np.array_equal(c._keep[1].cpu().numpy(), host.v)
+    kd = c._keep[0].cpu().numpy()
+    assert np.count_nonzero(kd != host.k) <= 4
+    # text rows
+    c1, c2 = p1a.KVCache.contiguous(kv_type, n_ctx, Hkv, D), p1a.KVCache.contiguous(kv_type, n_ctx, Hkv, D)
+    q1, q2 = torch.zeros_like(q), torch.zeros_like(q)
+    p1a.attn_prep(dev(qg), dev(k), dev(v), dev(qn), dev(kn), dev(pos), q1, gate, c1, -1, T, Hq, n_rot, base, eps)
+    p1a.attn_prep(dev(qg), dev(k), dev(v), dev(qn), dev(kn), dev(pos), q2, gate, c2, -1, T, Hq, n_rot, base, eps,
+                  mrope=(dev(np.stack([pos, pos, pos])), T, (11, 11, 10), 32))
+    torch.cuda.synchronize()
+    assert torch.equal(q1, q2) and torch.equal(c1._keep[0], c2._keep[0]) and torch.equal(c1._keep[1], c2._keep[1])
+    with pytest.raises(p1a.P1AError, match="M-RoPE"):
+        p1a.attn_prep(dev(qg), dev(k), dev(v), dev(qn), dev(kn), dev(pos), q2, gate, c2, -1, T, Hq, n_rot, base, eps,
+                      mrope=(dev(mp), T + 3, (11, 11, 10), 0))

@@ -162,3 +162,78 @@ def test_a16_quant_against_numpy_and_closed_forms():
     assert np.float32(vals[2, 0].astype(np.float32).max()) > 1.0      # |v| / 65504 passes 1 for the clamped group
     # every scaled value is v / amax: the largest magnitude of an ordinary group is exactly 1
     assert np.abs(vals[0, 0].astype(np.float32)).max() == 1.0
+
+
+# ---- interleaved M-RoPE (src/fast/mrope.cuh) ----
+# Which stream each rotary pair of the first 32 uses with the model's sections [11, 11, 10, 0] (sect 32), written out by
+# hand from the rule's words: streams interleave t, h, w, t, h, w, ... while their sections last (t and h 11 pairs each =
+# sectors below 33, w 10 pairs = sectors below 30), so sector 29 (29 % 3 == 2, but 29 < 30) is still w and nothing falls
+# to the fourth stream.
+STREAMS_11_11_10 = "thw" * 10 + "th"
+# sections [2, 1, 1, 0] (sect 4): sector 0 -> t; 1 -> h (1 < 3); 2 -> w (2 < 3); 3 -> 3 % 3 == 0 and 3 < 6 -> t
+STREAMS_2_1_1 = "thwt"
+
+
+def stream_table(sections, n):
+    s0, s1, s2, s3 = sections
+    sect = s0 + s1 + s2 + s3
+    tab = {(11, 11, 10, 0): STREAMS_11_11_10, (2, 1, 1, 0): STREAMS_2_1_1}[tuple(sections)]
+    return [tab[j % sect] for j in range(n)], sect
+
+
+def test_mrope_text_rows_are_plain_neox_bitwise():
+    """t = h = w = p: every pair rotates by p (src/fast/mrope.cuh:6-7)"""
+    Hq, Hkv, D, n_rot, T = 4, 1, 256, 64, 6
+    qg, k, v, qn, kn = make(11, T, Hq, Hkv, D)
+    pos = np.array([0, 3, 500, 501, 9000, 65000], np.int32)
+    for kt in TYPES:
+        c1, c2 = O.HostKV.contiguous(kt, 66000, Hkv, D), O.HostKV.contiguous(kt, 66000, Hkv, D)
+        q1, g1 = O.attn_prep(c1, qg, k, v, qn, kn, pos, -1, Hq, n_rot, 1e7)
+        q2, g2 = O.attn_prep(c2, qg, k, v, qn, kn, pos, -1, Hq, n_rot, 1e7, mrope=(np.stack([pos, pos, pos]), (11, 11, 10), 32))
+        assert np.array_equal(q1, q2) and np.array_equal(g1, g2)
+        assert np.array_equal(c1.k, c2.k) and np.array_equal(c1.v, c2.v)
+
+
+@pytest.mark.parametrize("sections,n_rot", [((11, 11, 10, 0), 64), ((2, 1, 1, 0), 32), ((11, 11, 10, 0), 128)])
+def test_mrope_each_pair_rotates_by_its_stream(sections, n_rot):
+    """against float64 with the stream of every pair taken from the hand-written tables"""
+    Hq, Hkv, D, T, base, eps = 2, 1, 128, 3, 1e6, 1e-6
+    qg, k, v, qn, kn = make(12, T, Hq, Hkv, D)
+    streams, sect = stream_table(sections, n_rot // 2)
+    mp = np.array([[7, 100, 2000], [9, 140, 2077], [30, 101, 1950]], np.int32)      # t, h, w of the 3 rows
+    pos = np.array([5, 6, 7], np.int32)                                              # cache rows: unrelated to the rotation
+    c = O.HostKV.contiguous(O.KV_F16, 16, Hkv, D)
+    q, _ = O.attn_prep(c, qg, k, v, qn, kn, pos, -1, Hq, n_rot, base, eps, mrope=(mp, sections[:3], sect))
+    half = n_rot // 2
+    for t in range(T):
+        x = qg[t, 0, :D].astype(np.float64)
+        y = x / np.sqrt((x * x).mean() + eps) * qn.astype(np.float64)
+        p = np.array([mp["thw".index(s), t] for s in streams], np.float64)
+        th = p * base ** (-2.0 * np.arange(half) / n_rot)
+        ref = y.copy()
+        ref[:half] = y[:half] * np.cos(th) - y[half:n_rot] * np.sin(th)
+        ref[half:n_rot] = y[:half] * np.sin(th) + y[half:n_rot] * np.cos(th)
+        assert np.max(np.abs(q[t, 0] - ref)) < (4e-6 + 2.0 * p.max() * 2.0 ** -24) * max(1.0, np.abs(ref).max())
+        # the K row landed at pos[t], rotated the same way
+        got = O.kv_read_head(c, 0, 0, int(pos[t]), 0)
+        xk = k[t, 0].astype(np.float64)
+        yk = xk / np.sqrt((xk * xk).mean() + eps) * kn.astype(np.float64)
+        refk = yk.copy()
+        refk[:half] = yk[:half] * np.cos(th) - yk[half:n_rot] * np.sin(th)
+        refk[half:n_rot] = yk[:half] * np.sin(th) + yk[half:n_rot] * np.cos(th)
+        assert np.max(np.abs(got - refk)) < 2e-3 * max(1.0, np.abs(refk).max())
+
+
+def test_mrope_moving_one_stream_moves_only_its_pairs():
+    Hq, Hkv, D, n_rot = 1, 1, 64, 64
+    qg, k, v, qn, kn = make(13, 1, Hq, Hkv, D)
+    streams, sect = stream_table((11, 11, 10, 0), 32)
+    base_p = np.array([[50], [50], [50]], np.int32)
+    c = O.HostKV.contiguous(O.KV_F16, 4, Hkv, D)
+    q0, _ = O.attn_prep(c, qg, k, v, qn, kn, np.array([0], np.int32), -1, Hq, n_rot, 1e4, mrope=(base_p, (11, 11, 10), sect))
+    for si, name in enumerate("thw"):
+        mp = base_p.copy()
+        mp[si, 0] = 61
+        q1, _ = O.attn_prep(c, qg, k, v, qn, kn, np.array([0], np.int32), -1, Hq, n_rot, 1e4, mrope=(mp, (11, 11, 10), sect))
+        changed = {j for j in range(32) if q1[0, 0, j] != q0[0, 0, j] or q1[0, 0, j + 32] != q0[0, 0, j + 32]}
+        assert changed == {j for j in range(32) if streams[j] == name}
