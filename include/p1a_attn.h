@@ -149,12 +149,13 @@ int p1a_ew_quant(int op, const float *a, const float *b, float *y, void *qbuf, i
  * fp16 MFMA products with fp32 accumulation; gate as in p1a_attn_decode. `scratch` is optional caller-supplied device
  * memory (256-byte aligned): with at least p1a_attn_prefill_scratch_bytes(...) bytes a q8_0 / q4_0 cache is converted to
  * f16 once per call instead of once per workgroup (same result bits, about 10-35 % less time); with less, or NULL, the
- * kernel converts on the fly.
+ * kernel converts on the fly. Rows of the cache past position p0 + T - 1 may be fetched (never past the end of a page,
+ * or of a contiguous cache) but are never weighted, whatever they hold.
  * Replaces attn_prefill (src/fast/attn.cuh:46-50) and attn_fold (src/fast/attn_fold.cuh:19-26).
  */
 int p1a_attn_prefill(const float *q, const p1a_kv *c, float *out, const float *gate, int T, int p0, int Hq,
                      float scale, void *scratch, size_t scratch_bytes, void *stream);
-/* bytes of scratch that enable the convert-once variant: 2 * (p0 + T) * Hkv * D * 2. Replaces attn_fold_scratch_bytes
+/* bytes of scratch that enable the convert-once variant: 2 * roundup(p0 + T, 16) * Hkv * D * 2. Replaces attn_fold_scratch_bytes
  * (src/fast/attn_fold.cuh:19). */
 size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D);
 

@@ -77,6 +77,7 @@ struct pf_params {
     const char * vc;
     kv_view pg;
     int T, p0, Hq, Hkv, GQA;
+    int n_rows;   // positions the cache holds (contiguous caches: rows that may be read)
     float qscale;
     int nblk;     // token blocks
 };
@@ -323,11 +324,14 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     constexpr bool FAST = GROUPED && IM::WAVE_MAJOR;
     struct gpages { int pg; };
     struct gbases { size_t go; };
+    // a group past the last position takes the base of the last one that holds a position: the LDS-direct loads then
+    // fetch that group's 16 rows (all inside its page) instead of clamping row by row
+    const int gclamp = DMA ? (pmax & ~15) : pmax;
     auto group_pages = [&](int tile) {
         gpages r;
         r.pg = 0;
         if (FAST && ptab) {
-            const int32_t * e = ptab + (__builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, pmax)) >> P.pg.psh);
+            const int32_t * e = ptab + (__builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, gclamp)) >> P.pg.psh);
             asm volatile("s_load_dword %0, %1, 0x0" : "=s"(r.pg) : "s"(e));
         }
         return r;
@@ -335,7 +339,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     auto group_bases = [&](int tile, gpages & gp) {
         gbases r;
         asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(gp.pg));
-        const int p = __builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, pmax));
+        const int p = __builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, gclamp));
         r.go = (ptab ? (size_t) gp.pg * P.pg.pstride + (size_t) (p & pmask) * P.pg.rowb : (size_t) p * P.pg.rowb) + head_off;
         return r;
     };
@@ -435,16 +439,19 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     };
 
     // ---- LDS-direct tile loads (DMA): wave w moves the 8 blocks of its 16-key group; instruction j takes keys j and
-    // j + 8 of the group (lanes 0-31 / 32-63, 16 bytes of the row each). In the tile that holds pmax the rows past it
-    // repeat the last written one ----
-    // (no branches: the two row numbers of a block are clamped in scalar registers, each lane picks its own)
-    const uint32_t dma_col = (uint32_t) (lane & 31) * 16u;
-    const int dma_room = __builtin_amdgcn_readfirstlane(max(pmax - (last_tile * BN + 16 * wave), 0));
-    auto dma_block = [&](const char * cache, int tile, const gbases & gb, char * dst_tile, int bstride, int j) {
-        const int room = tile == last_tile ? dma_room : 15;
-        const uint32_t r0 = __builtin_amdgcn_readfirstlane((uint32_t) min(j, room) * (uint32_t) P.pg.rowb);
-        const uint32_t r1 = __builtin_amdgcn_readfirstlane((uint32_t) min(j + 8, room) * (uint32_t) P.pg.rowb);
-        dma16(cache + gb.go, (g ? r1 : r0) + dma_col, lds_addr(dst_tile + (8 * wave + j) * bstride));
+    // j + 8 of the group (lanes 0-31 / 32-63, 16 bytes of the row each): a scalar base that advances by one row per
+    // instruction and ONE loop-invariant lane offset. Rows past the last position are fetched as they are (the group lies
+    // inside one page, or inside the cache when it is contiguous - the host checks): as K they only make scores that the
+    // mask replaces; as V they are overwritten with zeros in LDS once the tile has landed (P = 0 times anything finite).
+    const uint32_t dma_vo = (uint32_t) (8 * g) * (uint32_t) P.pg.rowb + (uint32_t) (lane & 31) * 16u;
+    auto dma_block = [&](const char * cache, const gbases & gb, char * dst_tile, int bstride, int j) {
+        dma16(cache + gb.go + (size_t) j * P.pg.rowb, dma_vo, lds_addr(dst_tile + (8 * wave + j) * bstride));
+    };
+    auto zero_v_tail = [&](int tile, char * vtile) {
+        if (tile != last_tile) return;
+        const int room = pmax - (last_tile * BN + 16 * wave);             // the wave's last key that exists (< 0: none)
+        for (int kg = max(room + 1, 0); kg < 16; ++kg)
+            *reinterpret_cast<u2v *>(vtile + L::key_off(16 * wave + kg, L::VB) + lane * 8) = u2v{0u, 0u};
     };
 
     // ---- prologue: K(0), V(0), K(1) in LDS; (staged through registers: V(1) and K(2) on their way); S^T(0) ----
@@ -458,12 +465,13 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         gb_prev = group_bases(tile_of(1), g1);
         gp_ahead = group_pages(tile_of(2));
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dma_block(P.kc, tile_of(0), b0, lds, L::KB, j);
+        for (int j = 0; j < 8; ++j) dma_block(P.kc, b0, lds, L::KB, j);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dma_block(P.vc, tile_of(0), b0, lds + L::KT_B, L::VB, j);
+        for (int j = 0; j < 8; ++j) dma_block(P.vc, b0, lds + L::KT_B, L::VB, j);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) dma_block(P.kc, tile_of(1), gb_prev, lds + L::STAGE_B, L::KB, j);
+        for (int j = 0; j < 8; ++j) dma_block(P.kc, gb_prev, lds + L::STAGE_B, L::KB, j);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        zero_v_tail(tile_of(0), lds + L::KT_B);
     } else {
         gpages g0 = group_pages(tile_of(0)), g1 = group_pages(tile_of(1)), g2 = group_pages(tile_of(2));
         const gbases b0 = group_bases(tile_of(0), g0), b1 = group_bases(tile_of(1), g1);
@@ -553,8 +561,8 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             if constexpr (DMA) {   // one tile load every other step: K(it+2) first (it is needed first), then V(it+1)
                 if (k % 2 == 0) {
                     const int j = k / 2;
-                    if (j < 8) dma_block(P.kc, tile_of(it + 2), gb_dma, st_cur, L::KB, j);
-                    else if (j < 16) dma_block(P.vc, tile_of(it + 1), gb_prev, st_nxt + L::KT_B, L::VB, j - 8);
+                    if (j < 8) dma_block(P.kc, gb_dma, st_cur, L::KB, j);
+                    else if (j < 16) dma_block(P.vc, gb_prev, st_nxt + L::KT_B, L::VB, j - 8);
                 }
             }
             const int u = k / C::NKS;
@@ -581,44 +589,39 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         }
 
         PT(2);
+        // ---- O^T += V^T(it) P^T: set-up. V(it) has been in LDS since the last barrier, so its first fragments are asked
+        // for ahead of the exchange: their latency hides behind it ----
+        // Slot e of lane half g in k-step ps is key 32 (ps / 2) + 8 (ps % 2) + 4 g + e (e < 4), or that + 16 for e - 4
+        const int i16 = lane & 15, blk = lane >> 4;        // 16-lane block: dims 16 (blk & 1) .., lane half blk >> 1 == g
+        const int kk = i16 >> 2, jq = i16 & 3;
+        const char * vbase = st_cur + L::KT_B + L::v_lane(4 * g + kk) + (16 * (blk & 1) + 4 * jq) * 2 + dh * HD * 64;
+        // per k-step: HD fragments of V^T, each multiplied with the own and the partner's P^T, then the denominator
+        constexpr int NFR = (BN / 16) * HD, PF_V = 3;
+        constexpr int NP = 2 * S::NPT * S::PARTS;                             // store parts: K items, then V items
+        struct vfrag { s4 lo, hi; };
+        auto vread = [&](int f) {
+            const char * p0_ = vbase + (f % HD) * 64;
+            return vfrag{__builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + L::v_lo(f / HD))),
+                         __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + L::v_hi(f / HD)))};
+        };
+        vfrag vf[NFR];
+#pragma unroll
+        for (int f = 0; f < PF_V && f < NFR; ++f) vf[f] = vread(f);
         // ---- hand P^T and the rescale factor of the own rows to the partner ----
 #pragma unroll
         for (int ps = 0; ps < BN / 16; ++ps) *reinterpret_cast<h8 *>(px_own + (ps * 64 + lane) * 16) = pb[ps];
         if (g == 0) ax_own[c] = alpha;
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        {
-            const float alpha_p = ax_par[c];
-            if (__builtin_expect(__any(alpha_p != 1.0f), 0)) {
-#pragma unroll
-                for (int i = 0; i < 16; ++i)
-#pragma unroll
-                    for (int dt = 0; dt < HD; ++dt) o[1][dt][i] *= alpha_p;
-            }
-        }
         PT(6);
-        // ---- stream 1: O^T += V^T(it) P^T on the matrix pipe; stream 2: K(it+2), V(it+1) -> f16 tiles in LDS ----
+        // ---- stream 1: O^T += V^T(it) P^T on the matrix pipe; stream 2: masking and row maximum of S^T(it+1) (and K(it+2),
+        // V(it+1) -> f16 tiles in LDS when they are staged through registers) ----
         {
-            // Slot e of lane half g in k-step ps is key 32 (ps / 2) + 8 (ps % 2) + 4 g + e (e < 4), or that + 16 for e - 4
-            const int i16 = lane & 15, blk = lane >> 4;        // 16-lane block: dims 16 (blk & 1) .., lane half blk >> 1 == g
-            const int kk = i16 >> 2, jq = i16 & 3;
-            const char * vbase = st_cur + L::KT_B + L::v_lane(4 * g + kk) + (16 * (blk & 1) + 4 * jq) * 2 + dh * HD * 64;
-            // per k-step: HD fragments of V^T, each multiplied with the own and the partner's P^T, then the denominator
-            constexpr int NFR = (BN / 16) * HD, PF_V = 3;
-            constexpr int NP = 2 * S::NPT * S::PARTS;                             // store parts: K items, then V items
-            struct vfrag { s4 lo, hi; };
-            auto vread = [&](int f) {
-                const char * p0_ = vbase + (f % HD) * 64;
-                return vfrag{__builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + L::v_lo(f / HD))),
-                             __builtin_amdgcn_ds_read_tr16_b64_v4i16((s4 __attribute__((address_space(3))) *) (p0_ + L::v_hi(f / HD)))};
-            };
-            vfrag vf[NFR];
+            const float alpha_p = ax_par[c];                                      // (needed before the partner's first product)
             h8 pp[BN / 16];
             constexpr int MPS = 32 / NFR;                                          // next tile's values masked per step
             static_assert(32 % NFR == 0, "mask slices must tile the 32 values of a lane");
             const int k0n = tile_of(it + 1) * BN;
             mloc = NEG_INF;
-#pragma unroll
-            for (int f = 0; f < PF_V && f < NFR; ++f) vf[f] = vread(f);
             pp[0] = *reinterpret_cast<const h8 *>(px_par + lane * 16);
 #pragma unroll
             for (int f = 0; f < NFR; ++f) {
@@ -628,6 +631,12 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                 const h4 l4 = __builtin_bit_cast(h4, vf[f].lo), h4_ = __builtin_bit_cast(h4, vf[f].hi);
                 const h8 a = {l4[0], l4[1], l4[2], l4[3], h4_[0], h4_[1], h4_[2], h4_[3]};
                 o[0][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[ps], o[0][dt], 0, 0, 0);
+                if (f == 0 && __builtin_expect(__any(alpha_p != 1.0f), 0)) {       // the partner's rows moved their reference maximum
+#pragma unroll
+                    for (int i = 0; i < 16; ++i)
+#pragma unroll
+                        for (int d2 = 0; d2 < HD; ++d2) o[1][d2][i] *= alpha_p;
+                }
                 o[1][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pp[ps], o[1][dt], 0, 0, 0);
                 if (dt == HD - 1) ol = __builtin_amdgcn_mfma_f32_32x32x16_f16(ones, pb[ps], ol, 0, 0, 0);
 #pragma unroll
@@ -649,6 +658,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         if constexpr (DMA) {
             gb_prev = gb_dma;
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        // this step's tile loads have landed
+            zero_v_tail(tile_of(it + 1), st_nxt + L::KT_B);
         } else {
             const gbases gb_k = group_bases(tile_of(it + 3), gp_k);
             load_tile(rk, P.kc, tile_of(it + 3), gb_k);
@@ -717,7 +727,9 @@ int launch_pf(const pf_params & P, hipStream_t s) {
     if constexpr (KT == P1A_KV_F16 && D == 256) {
         static const bool no_dma = getenv("P1A_PF_NODMA") && atoi(getenv("P1A_PF_NODMA"));   // development A/B switch
         // (rows of whole 16-byte units at 16-byte aligned addresses: what a 16-byte load per lane needs)
-        if (grouped && !no_dma && P.pg.rowb % 16 == 0 && P.pg.rowb * 16 < (1ull << 32)) return launch_pf_g<KT, D, true, true>(P, s);
+        // and whole 16-key groups that can be read: always inside a page; inside a contiguous cache when it holds them
+        const bool groups_ok = P.pg.pt || ((P.p0 + P.T - 1) | 15) < P.n_rows;
+        if (grouped && !no_dma && groups_ok && P.pg.rowb % 16 == 0 && P.pg.rowb * 16 < (1ull << 32)) return launch_pf_g<KT, D, true, true>(P, s);
     }
     return grouped ? launch_pf_g<KT, D, true>(P, s) : launch_pf_g<KT, D, false>(P, s);
 }
@@ -774,7 +786,8 @@ __global__ void __launch_bounds__(256) dq_k(const char * kc, const char * vc, kv
 }   // namespace
 
 // bytes of the f16 staging copy of the first n positions (K and V)
-size_t prefill_stage_bytes(int n, int Hkv, int D) { return 2 * (size_t) n * Hkv * D * 2; }
+// (rows rounded up to whole 16-key groups: the attention kernel fetches whole groups)
+size_t prefill_stage_bytes(int n, int Hkv, int D) { return 2 * (size_t) ((n + 15) & ~15) * Hkv * D * 2; }
 
 int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s) {
@@ -783,6 +796,7 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
     pf_params P;
     P.q = q; P.out = out; P.gate = gate; P.kc = (const char *) c.k; P.vc = (const char *) c.v; P.pg = view_of(c);
     P.T = T; P.p0 = p0; P.Hq = Hq; P.Hkv = c.Hkv; P.GQA = Hq / c.Hkv;
+    P.n_rows = c.n_ctx;
     P.qscale = scale * 1.4426950408889634f;
     P.nblk = (T + BM - 1) / BM;
 #define PF(KT_) (c.D == 256 ? launch_pf<KT_, 256>(P, s) : c.D == 128 ? launch_pf<KT_, 128>(P, s) : launch_pf<KT_, 64>(P, s))
@@ -793,7 +807,8 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
     const int n = p0 + T;
     static const bool no_stage = getenv("P1A_PF_NOSTAGE") && atoi(getenv("P1A_PF_NOSTAGE"));   // development A/B switch
     if (!no_stage && scratch && !((uintptr_t) scratch & 255) && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D)) {
-        char * ko = (char *) scratch, * vo = ko + (size_t) n * c.Hkv * c.D * 2;
+        const int n16 = (n + 15) & ~15;
+        char * ko = (char *) scratch, * vo = ko + (size_t) n16 * c.Hkv * c.D * 2;
         const long long items = (long long) n * (c.Hkv * c.D / (c.type == P1A_KV_Q8_0 ? 16 : 32));
         const unsigned blocks = (unsigned) ((items + 255) / 256);
         if (c.type == P1A_KV_Q8_0) dq_k<P1A_KV_Q8_0><<<blocks, 256, 0, s>>>(P.kc, P.vc, P.pg, n, c.Hkv, c.D, ko, vo);
@@ -802,6 +817,7 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
         P.kc = ko; P.vc = vo;
         P.pg.pt = nullptr; P.pg.rtab = nullptr; P.pg.psh = 0; P.pg.pstride = 0;
         P.pg.rowb = (size_t) c.Hkv * c.D * 2;
+        P.n_rows = n16;
         return PF(P1A_KV_F16);
     }
     if (c.type == P1A_KV_Q8_0) return PF(P1A_KV_Q8_0);

@@ -93,11 +93,42 @@ def test_scratch_variant_gives_the_same_bits(p1a, kv_type, Hq, Hkv, D, psh):
     q, _, _, gate = I.qkv(70 + D, 1, T, Hq, Hkv, D, f16_inputs=True)
     a = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16, gate=gate)
     need = p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D)
-    assert need == 2 * (p0 + T) * Hkv * D * 2
+    assert need == 2 * ((p0 + T + 15) // 16 * 16) * Hkv * D * 2       # whole 16-key groups of f16 rows, K and V
     dq, dg = dev(q), dev(gate)
     for nbytes in (need, need // 2):
-        scr = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
+        scr = torch.full((nbytes,), 0xff, dtype=torch.uint8, device="cuda")   # (what the copy does not write is NaN)
         out = torch.zeros((T, Hq, D), device="cuda")
         p1a.attn_prefill(dq, pool.dev_seq(0), out, T, p0, Hq, 1 / 16, gate=dg, scratch=scr)
         torch.cuda.synchronize()
         assert np.array_equal(out.cpu().numpy(), a), nbytes
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("p0,T", [(0, 37), (50, 130), (128, 1)])
+def test_rows_past_the_last_position_are_never_weighted(p1a, kv_type, p0, T):
+    """whatever lies in the cache past the last position - here NaN / Inf bit patterns - must not reach the output (the
+    kernels may fetch such rows with a tile; they must not let them count)"""
+    Hq, Hkv, D, psh = 12, 2, 256, 6
+    n = p0 + T
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n, 40], seed=41, n_layers=1, layer=0)
+    q, _, _, gate = I.qkv(91, 1, T, Hq, Hkv, D, f16_inputs=True)
+    want = O.attn_rows(pool.host_seq(0), q, np.arange(p0, p0 + T), Hq, 1 / 16, gate=gate)
+    # poison every row of the sequence's last page past position n - 1, K and V
+    c = pool.dev_seq(0)
+    rb = O.row_bytes(kv_type, Hkv, D)
+    ps = 1 << psh
+    page = int(pool.tabs[(n - 1) >> psh])
+    first = ((n - 1) & (ps - 1)) + 1
+    if first < ps:
+        for base in (0, ps * rb):                                  # K block, V block of the page (one layer)
+            o = page * c.pstride + base + first * rb
+            pool.dpool[o:o + (ps - first) * rb] = 0xff if kv_type != O.KV_F16 else 0x7e
+    out = run_prefill(p1a, c, q, T, p0, Hq, 1 / 16, gate=gate)
+    assert np.isfinite(out).all()
+    ma, rl = I.errors(out, want)
+    assert ma < 2e-3 and rl < 1e-3, (ma, rl)
+    scr = torch.full((p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D),), 0xff, dtype=torch.uint8, device="cuda")
+    out2 = torch.full((T, Hq, D), float("nan"), device="cuda")
+    p1a.attn_prefill(dev(q), c, out2, T, p0, Hq, 1 / 16, gate=dev(gate), scratch=scr)
+    torch.cuda.synchronize()
+    assert np.array_equal(out2.cpu().numpy(), out)
