@@ -132,3 +132,27 @@ def test_rows_past_the_last_position_are_never_weighted(p1a, kv_type, p0, T):
     p1a.attn_prefill(dev(q), c, out2, T, p0, Hq, 1 / 16, gate=dev(gate), scratch=scr)
     torch.cuda.synchronize()
     assert np.array_equal(out2.cpu().numpy(), out)
+
+
+def test_f16_contiguous_and_small_pages_take_the_same_bits(p1a):
+    """f16, D = 256: a contiguous cache that ends right behind the last position (whole 16-key groups cannot be fetched:
+    the register-staged kernel runs), one with room (tiles loaded straight into LDS) and 16-position pages must agree
+    bit for bit, and with the oracle within the tolerance"""
+    Hq, Hkv, D, p0, T = 12, 2, 256, 203, 170
+    n = p0 + T                                                 # 373: not a multiple of 16
+    q, k, v, gate = I.qkv(55, n, T, Hq, Hkv, D, f16_inputs=True)
+    host = O.HostKV.contiguous(O.KV_F16, n, Hkv, D)
+    O.kv_append_rows(host, k, v, np.arange(n))
+    want = O.attn_rows(host.view(), q, np.arange(p0, n), Hq, 1 / 16, gate=gate)
+    outs = []
+    for n_ctx in (n, n + 40):
+        c = p1a.KVCache.contiguous(O.KV_F16, n_ctx, Hkv, D)
+        p1a.kv_append(c, dev(k), dev(v), 0, n)
+        outs.append(run_prefill(p1a, c, q, T, p0, Hq, 1 / 16, gate=gate))
+    pool = Pool(p1a, O.KV_F16, Hq, Hkv, D, 4, [n, 30], seed=55, n_layers=2, layer=1, fill="none")
+    c = pool.dev_seq(0)
+    p1a.kv_append(c, dev(k), dev(v), 0, n)
+    outs.append(run_prefill(p1a, c, q, T, p0, Hq, 1 / 16, gate=gate))
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+    ma, rl = I.errors(outs[0], want)
+    assert ma < 2e-3 and rl < 1e-3, (ma, rl)
