@@ -23,6 +23,8 @@
 // so they stream the same K/V tiles through one L2.
 #include "p1a_common.hpp"
 
+#include <atomic>
+
 namespace p1a {
 size_t prefill_stage_bytes(int n, int Hkv, int D);
 namespace {
@@ -707,14 +709,18 @@ template <uint32_t KT, int D, bool GROUPED, bool DMA = false>
 int launch_pf_g(const pf_params & P, hipStream_t s) {
     using L = pf_lay<D>;
     const int lds = 2 * L::STAGE_B + (stager<KT, D>::SCALES_VIA_LDS ? 2 * 4 * 16 * stager<KT, D>::SB : 0) + 4 * (BN / 16) * 64 * 16 + 4 * 32 * 4;
-    static bool attr_set = false;
-    if (!attr_set) {
+    // (the attribute belongs to the function on ONE device: remembered per device, set again on another)
+    static std::atomic<uint32_t> attr_set{0};
+    int dev = 0;
+    (void) hipGetDevice(&dev);
+    const uint32_t bit = 1u << (dev & 31);
+    if (!(attr_set.load(std::memory_order_acquire) & bit)) {
         if (hipFuncSetAttribute((const void *) prefill_k<KT, D, GROUPED, DMA>, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
             (void) hipGetLastError();
             set_error("p1a_attn_prefill: cannot reserve %d bytes of LDS", lds);
             return P1A_E_LAUNCH;
         }
-        attr_set = true;
+        attr_set.fetch_or(bit, std::memory_order_release);
     }
     const int units = P.nblk * P.Hkv;
     const int slots = ((units + 7) / 8) * P.GQA;
