@@ -248,11 +248,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             const int d0 = KT == P1A_KV_F16 ? 32 * m + 8 * g : KT == P1A_KV_Q8_0 ? 16 * (4 * (m >> 1) + g) + 8 * (m & 1) : 32 * m + 4 * g;
             const int d1 = KT == P1A_KV_Q4_0 ? d0 + 16 : d0 + 4;
             float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-#ifndef P1A_EXP_NOQ
             if (livec) { a = *reinterpret_cast<const float4 *>(qr + d0); b = *reinterpret_cast<const float4 *>(qr + d1); }
-#else
-            a.x = (float) (size_t) qr;
-#endif
             const float s = P.qscale;
             qf[r][m] = h8{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s),
                           (half_t) (b.x * s), (half_t) (b.y * s), (half_t) (b.z * s), (half_t) (b.w * s)};
@@ -287,10 +283,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 #pragma unroll
         for (int r = 0; r < NT; ++r) s[r] = f4{0.f, 0.f, 0.f, 0.f};
         const char * krow = ks + c * C::HB;
-#ifdef P1A_EXP_NOQK
-        s[0][0] = *reinterpret_cast<const float *>(krow);
-        if (false)
-#endif
         if constexpr (KT == P1A_KV_F16) {
 #pragma unroll
             for (int m = 0; m < C::NMF; ++m) {
@@ -374,10 +366,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 
         if (have_n) wait_vm_imm<C::NRND>(); else wait_vm_imm<0>();   // V of tile t has landed (only K of t + 1 is younger)
         // ---- O^T += V^T P^T: k-slot i of lane group g is key ts + 4 g + i, the key of this lane's P value i ----
-#ifdef P1A_EXP_NOPV
-        o[0][0][0] += *reinterpret_cast<const float *>(vs + lane * 4);
-        if (false)
-#endif
         if constexpr (KT == P1A_KV_F16) {
             const int kk = c >> 2, jq = c & 3;
             const char * vr0 = vs + (4 * g + kk) * C::HB + jq * 8;
@@ -463,9 +451,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         if (tile_start(t + 1) < n_max) step(ks1, vs1, ks0, vs0, t + 1);
     }
     TS(12);
-#ifdef P1A_EXP_NOEPI
-    if (m_run[0] != 12345.f) return;
-#endif
 
     // ---- fold the WPH waves of each head (in sub order) and write one partial per (workgroup, head); the 16
     // columns of one MFMA tile at a time, so that a column is merged the same way whatever NT is. A wave parks its
@@ -512,23 +497,12 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             const int col = 16 * r + cc;
             const int t = col / P.GQA, hh = col - t * P.GQA;
             const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) (hg * P.HPW + hs) * P.GQA + hh;
-#if defined(P1A_EXP_NOSTORE)
-            if (M == 12345.f) *reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4) = acc;
-#elif defined(P1A_EXP_NTSTORE)
-            if (M != NEG_INF) __builtin_nontemporal_store(acc, reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4));
-            if (d4 == 0) {
-                float * pm = P.part_ml + (row * P.nsplit + split) * 2;
-                __builtin_nontemporal_store(M, pm);
-                __builtin_nontemporal_store(l, pm + 1);
-            }
-#else
             if (M != NEG_INF) *reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4) = acc;
             if (d4 == 0) {
                 float * pm = P.part_ml + (row * P.nsplit + split) * 2;
                 pm[0] = M;
                 pm[1] = l;
             }
-#endif
         }
     }
     TS(13);
