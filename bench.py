@@ -163,6 +163,21 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
     ex["batched_8slots_q8_0_us"] = round(sec * 1e6, 2)
     ex["batched_GBs"] = round(bb / sec / 1e9, 1)
     ex["batched_ctx"] = lens
+    del kv, cr
+    # the same kernel with enough to stream: 4 sequences of 65536 tokens, one row each, q8_0 (570 MB of KV per call)
+    n4 = 65536
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, n4, 4, seed=24)
+    pos = torch.full((4,), n4 - 1, dtype=torch.int32, device="cuda")
+    rt = torch.tensor([s * ppseq for s in range(4)], dtype=torch.int32, device="cuda")
+    q = normed((4, Hq, D))
+    gate = torch.randn((4, Hq * D), generator=g, device="cuda")
+    out = torch.empty((4, Hq, D), device="cuda")
+    cr = kv.with_rows(rt)
+    with torch.cuda.stream(stream):
+        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 4, pos, Hq, scale, gate=gate)] * 10, 2)
+    lb = 4 * n4 * 2 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
+    ex["decode_4x64K_q8_0_us"] = round(sec * 1e6, 2)
+    ex["decode_4x64K_GBs"] = round(lb / sec / 1e9, 1)
     return ex
 
 
