@@ -68,6 +68,7 @@ struct dec_params {
     int T, RG, Hq, Hkv, GQA, HPW;
     float qscale;     // softmax scale * log2(e)
     int nsplit;       // split streams
+    int spw;          // split streams one workgroup walks, one after the other (nsplit % spw == 0)
 };
 
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
@@ -125,7 +126,7 @@ __device__ __forceinline__ int sload_i32(const int32_t * p) {
 }
 __device__ __forceinline__ void wait_scalar(int & v) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(v)); }
 
-template <uint32_t KT, int D, int NT, int NWV>
+template <uint32_t KT, int D, int NT, int NWV, bool MULTI>
 __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
     // four tile slots per wave (K and V, two each) as separate arrays, plus a small per-wave table
@@ -140,9 +141,14 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     const int c = lane & 15, g = lane >> 4;
     // blockIdx.x -> (split stream, head group). Workgroups are dealt to the 8 XCDs round-robin by linear index, so
     // the head groups of one split stream (which share cache lines when HPW < Hkv) are given the same index mod 8.
+    // A workgroup may walk several split streams in turn (spw > 1, when a call has many more workgroups than the device
+    // has CUs): stream split, split + nsplit / spw, ... - every stream is computed and written exactly as if it had a
+    // workgroup of its own, only the per-workgroup set-up is shared.
     const int HG = P.Hkv / P.HPW;
+    const int spw = MULTI ? P.spw : 1;
+    const int nwgs = P.nsplit / spw;                          // workgroup-streams
     int split, hg;
-    if ((P.nsplit & 7) == 0) {
+    if ((nwgs & 7) == 0) {
         const int i = blockIdx.x, j = i >> 3;
         hg = j % HG;
         split = (j / HG) * 8 + (i & 7);
@@ -220,6 +226,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 
     // first requests: K then V of tile 0; every later tile is requested, one load at a time, from inside the step
     // before it, so that a wave is never parked on the memory pipeline for long while it has products to compute
+    auto first_requests = [&]() {
     const bool have0 = tile_start(0) < n_max;
     if (have0) {
         int pg0 = 0;
@@ -231,6 +238,8 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 #pragma unroll
         for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vs0, P.vc + o0, tile_start(0), rd);
     }
+    };
+    first_requests();
     TS(1);
 
     // Q^T operands: column = query row (token t, head hh of the group), 8 consecutive dims per MFMA slot group
@@ -258,6 +267,13 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     f4 o[NT][C::NDT];
     f4 ol[NT];
     float m_run[NT];
+    const h4 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
+    for (int sw = 0; sw < spw; ++sw) {
+    if (MULTI && sw) {                                                 // the next stream: the slots are free behind this barrier
+        __syncthreads();
+        split += nwgs;
+        first_requests();
+    }
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         m_run[r] = NEG_INF;
@@ -265,7 +281,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 #pragma unroll
         for (int j = 0; j < C::NDT; ++j) o[r][j] = f4{0.f, 0.f, 0.f, 0.f};
     }
-    const h4 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
 
     // one 16-key tile from slots (ks, vs); the loads of tile t + 1 into (ksn, vsn) are issued between its products
     auto step = [&](char * ks, char * vs, char * ksn, char * vsn, int t) {
@@ -505,6 +520,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             }
         }
     }
+    }   // streams of this workgroup
     TS(13);
 }
 
@@ -686,6 +702,7 @@ struct dec_plan {
     int GQA, HPW, NW, NT, RG;
     int nsplit;    // split streams
     int NS;        // partials per output row (what merge_k folds)
+    int spw;       // split streams per workgroup
 };
 
 bool mfma_ok(const p1a_kv & c, int GQA) {
@@ -739,6 +756,19 @@ void finish_plan(dec_plan & p) {
     if (p.mfma) p.NS = p.nsplit;
 }
 
+// how many split streams a workgroup walks: 1 until the call has more than four workgroups per CU slot; then as many
+// as bring it back there (a power of two that divides nsplit; measured: 8 slots of unequal depth 89 -> 80 us at 2,
+// 91 us at 4 - fewer, longer workgroups balance worse). The partials do not depend on it.
+int streams_per_wg(const dec_plan & p, int Hkv, int T, int cus) {
+    static const int env = env_int("P1A_DEC_SPW", 0);         // development A/B knob
+    const long long wgs = (long long) p.nsplit * (Hkv / p.HPW) * ((T + p.RG - 1) / p.RG);
+    const int per_round = (p.NW == 8 ? 1 : 2) * cus;
+    int spw = 1;
+    while (spw * 2 <= p.nsplit && p.nsplit % (spw * 2) == 0 && wgs / spw > 4LL * per_round) spw *= 2;
+    if (env > 0 && p.nsplit % env == 0) spw = env;
+    return spw;
+}
+
 template <uint32_t KT, int D>
 int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hipStream_t s) {
     dec_params P;
@@ -747,17 +777,21 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     P.p0 = a.p0; P.p0_dev = a.p0_dev; P.pos_rows = a.pos_rows;
     P.T = a.T; P.RG = pl.RG; P.Hq = a.Hq; P.Hkv = c.Hkv; P.GQA = pl.GQA; P.HPW = pl.HPW;
     P.qscale = a.scale * 1.4426950408889634f; P.nsplit = pl.nsplit;
-    const dim3 grid(pl.nsplit * (c.Hkv / pl.HPW), (a.T + pl.RG - 1) / pl.RG);
+    P.spw = streams_per_wg(pl, c.Hkv, a.T, a.cus > 0 ? a.cus : 256);
+    const dim3 grid(pl.nsplit / P.spw * (c.Hkv / pl.HPW), (a.T + pl.RG - 1) / pl.RG);
     constexpr bool big_tiles = KT == P1A_KV_F16 && D == 256;
+#define P1A_DEC(NT_, NW_) do { if (P.spw > 1) dec_mfma_k<KT, D, NT_, NW_, true><<<grid, NW_ * 64, 0, s>>>(P); \
+                               else dec_mfma_k<KT, D, NT_, NW_, false><<<grid, NW_ * 64, 0, s>>>(P); } while (0)
     if (pl.NW == 8) {
         if constexpr (!big_tiles) {
-            if (pl.NT == 1) dec_mfma_k<KT, D, 1, 8><<<grid, 512, 0, s>>>(P);
-            else dec_mfma_k<KT, D, 2, 8><<<grid, 512, 0, s>>>(P);
+            if (pl.NT == 1) P1A_DEC(1, 8);
+            else P1A_DEC(2, 8);
         }
     } else {
-        if (pl.NT == 1) dec_mfma_k<KT, D, 1, 4><<<grid, 256, 0, s>>>(P);
-        else dec_mfma_k<KT, D, 2, 4><<<grid, 256, 0, s>>>(P);
+        if (pl.NT == 1) P1A_DEC(1, 4);
+        else P1A_DEC(2, 4);
     }
+#undef P1A_DEC
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 

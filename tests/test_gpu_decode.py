@@ -118,6 +118,13 @@ def test_config3_batched_slots(p1a):
     out = torch.empty((8, Hq, D), device="cuda")
     p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, 8, dev(pos), Hq, 1 / 16, gate=dev(gate))
     check(out.cpu().numpy(), ref, "config 3 (reduced)")
+    # a call this wide lets a workgroup walk several split streams; every row must still be bit for bit the row of a call
+    # of its own (one stream per workgroup)
+    for t in range(8):
+        one = torch.empty((1, Hq, D), device="cuda")
+        p1a.attn_decode_rows(dev(q[t:t + 1]), pool.devkv.with_rows(dev(rtab[t:t + 1])), one, 1, dev(pos[t:t + 1]), Hq, 1 / 16,
+                             gate=dev(gate[t:t + 1]))
+        assert torch.equal(one[0], out[t]), t
 
 
 @pytest.mark.parametrize("kv_type", [O.KV_Q4_0, O.KV_Q8_0])
