@@ -105,8 +105,7 @@ def test_bitwise_invariances(p1a, kv_type):
 
 
 def test_config3_batched_slots(p1a):
-    """8 slots sharing one paged q8_0 pool, lengths log-uniform in [1024, 32768] (scaled down 8x here; the full size
-    runs in test_full_size_configs), page tables interleaved, one row per slot"""
+    """8 slots sharing one paged q8_0 pool, lengths log-uniform in [1024, 32768] (scaled down 8x here; test_gpu_full_size.py runs the full size), page tables interleaved, one row per slot"""
     Hq, Hkv, D, psh = 24, 4, 256, 8
     g = I.rng(33)
     lens = [int(np.exp(g.uniform(np.log(128), np.log(4096)))) for _ in range(8)]
