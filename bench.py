@@ -356,6 +356,20 @@ def main():
                   "kernel_same_pool_GBs": round(step_bytes / sec_kernel_same / 1e9, 1),
                   "merge_kernel_us": round((sec - sec_kernel) * 1e6, 2), "nsplit": p1a.get_nsplit(Hkv)},
     }
+    # a reference point for the size: a library reduction (read-only stream) over the same number of bytes, rotating over
+    # buffers larger than the Infinity Cache - what the memory system gives a 71 MB launch that computes next to nothing
+    ref_bufs = [torch.ones(step_bytes // 4, device="cuda") for _ in range(n_pools)]
+    ref_out = torch.empty((), device="cuda")
+    it_ref = [0]
+
+    def ref_step():   # (eager, not captured: the library's reduction clears its own scratch memory)
+        it_ref[0] += 1
+        torch.sum(ref_bufs[it_ref[0] % n_pools], dim=0, out=ref_out)
+
+    sec_ref = time_eager(torch, ref_step, reps=64, warmup=8)
+    res["extra"]["stream_read_same_bytes_us"] = round(sec_ref * 1e6, 2)
+    res["extra"]["stream_read_same_bytes_GBs"] = round(step_bytes / sec_ref / 1e9, 1)
+    del ref_bufs
     if args.calib_copy:
         src = torch.ones(64 * 1024 * 1024, device="cuda")
         dst = torch.empty_like(src)
