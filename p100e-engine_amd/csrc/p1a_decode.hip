@@ -31,6 +31,7 @@ namespace p1a {
 namespace {
 
 constexpr float NEG_INF = -__builtin_inff();
+constexpr float RESCALE_STEP = 8.0f;   // log2 of the largest P the running maximum lets through
 
 template <uint32_t KT, int D> struct tile_cfg {
     static constexpr int HB = (int) head_bytes(KT, D);
@@ -87,6 +88,14 @@ __device__ __forceinline__ u2 deq4(uint32_t w, h2 d01, h2 d23) {
     const h2 a = __builtin_bit_cast(h2, perm(0x64646464u, x, 0x04010400u));
     const h2 b = __builtin_bit_cast(h2, perm(0x64646464u, x, 0x04030402u));
     return u2{__builtin_bit_cast(uint32_t, (a - off) * d01), __builtin_bit_cast(uint32_t, (b - off) * d23)};
+}
+
+// the maximum over the four lanes that share (lane & 15): the two 16-lane rows of each half, then the two halves
+__device__ __forceinline__ float max_over_groups(float m) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, m), __builtin_bit_cast(unsigned, m), false, false);
+    m = fmaxf(__builtin_bit_cast(float, a[0]), __builtin_bit_cast(float, a[1]));
+    const auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, m), __builtin_bit_cast(unsigned, m), false, false);
+    return fmaxf(__builtin_bit_cast(float, b[0]), __builtin_bit_cast(float, b[1]));
 }
 
 // 4 nibbles (the low nibbles of the 4 bytes of w) -> ((n - 8) * d) as two packed f16 pairs (0x6400 | n = 1024 + n)
@@ -231,7 +240,9 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     if (have0) {
         int pg0 = 0;
         if (ptab) pg0 = sload_i32(page_of(tile_start(0)));
+        TS(8);
         wait_scalar(pg0);
+        TS(9);
         const size_t o0 = tile_off(tile_start(0), pg0);
 #pragma unroll
         for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ks0, P.kc + o0, tile_start(0), rd);
@@ -264,6 +275,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         }
     }
 
+    TS(2);
     f4 o[NT][C::NDT];
     f4 ol[NT];
     float m_run[NT];
@@ -290,6 +302,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         int pgn = 0;
         if (ptab && have_n) pgn = sload_i32(page_of(tn));
         wait_vm_imm<C::NRND>();                               // K of tile t has landed (only its V is younger)
+        if (t == 0) TS(3); else if (t == 3) TS(4);
         wait_scalar(pgn);
         const size_t on = have_n ? tile_off(tn, pgn) : 0;
         const char * const kn = P.kc + on, * const vn = P.vc + on;
@@ -357,9 +370,10 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
                 else if (plim[r] < 0) s[r][i] = NEG_INF;
                 mloc = fmaxf(mloc, s[r][i]);
             }
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 16));
-            mloc = fmaxf(mloc, __shfl_xor(mloc, 32));
-            const float mnew = fmaxf(m_run[r], mloc);
+            mloc = max_over_groups(mloc);
+            // the running maximum only moves when a tile exceeds it by more than 2^RESCALE_STEP: P stays below that
+            // (f16 holds it, the sums are fp32) and the accumulators are rescaled far less often
+            const float mnew = mloc > m_run[r] + RESCALE_STEP ? mloc : m_run[r];
             const bool dead = mnew == NEG_INF;
             // nothing accumulated yet (m = -inf): the accumulators are zero and need no rescale
             alpha[r] = (dead || m_run[r] == NEG_INF) ? 1.0f : __builtin_amdgcn_exp2f(m_run[r] - mnew);
@@ -465,7 +479,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         step(ks0, vs0, ks1, vs1, t);
         if (tile_start(t + 1) < n_max) step(ks1, vs1, ks0, vs0, t + 1);
     }
-    TS(12);
+    TS(5);
 
     // ---- fold the WPH waves of each head (in sub order) and write one partial per (workgroup, head); the 16
     // columns of one MFMA tile at a time, so that a column is merged the same way whatever NT is. A wave parks its
@@ -488,6 +502,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             }
         }
         __syncthreads();
+        if (r == 0) TS(6);
         const int items = P.HPW * Rr * (D / 4);
         for (int it = threadIdx.x; it < items; it += NWV * 64) {
             const int d4 = it % (D / 4), rest = it / (D / 4);
@@ -521,7 +536,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         }
     }
     }   // streams of this workgroup
-    TS(13);
+    TS(7);
 }
 
 // ---- generic path: any D % 32 == 0 (<= 512), any GQA, every type; one wave per (split stream, q head, row) ----
