@@ -3,8 +3,8 @@
 // Work decomposition
 //   grid = (nsplit * head groups, row groups), block = NW waves (8, or 4 when a tile is large). A row group is up to
 //   4 query rows of ONE sequence (the tokens of a verify block); its GQA * rows query rows are the columns of 16-wide
-//   MFMA tiles, so the group's KV is read once. Wave w owns kv head (w % HPW) of the workgroup's head group and key
-//   sub-range (w / HPW): in unit u (32 * NW / HPW positions) it owns 32 consecutive positions, which it walks as two
+//   MFMA tiles, so the group's KV is read once. A workgroup owns one kv head; in unit u (32 * NW positions) wave w owns
+//   the 32 consecutive positions 32 w .., which it walks as two
 //   16-key tiles; split stream s owns the units s, s + nsplit, ... . The partition depends only on the device and
 //   Hkv, never on T, the depth or the batch, so a row is computed by the same sequence of operations whichever call
 //   it is part of (T-invariance, rows == single, paged == contiguous).
@@ -43,6 +43,7 @@ template <uint32_t KT, int D> struct tile_cfg {
     static constexpr int SLOT_B = TILE_B > QTR_B ? TILE_B : QTR_B;   // one LDS slot
     static constexpr int VA_B = KT == P1A_KV_Q4_0 ? 16 * 144 : 0;    // q4_0: 8-byte aligned copy of a V tile's nibbles
     static constexpr int TAB_B = 256;                          // per wave: transposed V scales, later (m, l) of the merge
+    static constexpr int QRS = D * 4 + 16;                     // row stride of the Q staging copy (padded: no bank conflicts)
     static constexpr int NMF = D / 32;                         // QK MFMAs per tile
     static constexpr int NDT = D / 16;                         // output dim tiles
     static_assert(HB % 16 == 0, "head row must be a whole number of 16-byte chunks");
@@ -66,7 +67,7 @@ struct dec_params {
     int p0;
     const int32_t * p0_dev;
     const int32_t * pos_rows;
-    int T, RG, Hq, Hkv, GQA, HPW;
+    int T, RG, Hq, Hkv, GQA;
     float qscale;     // softmax scale * log2(e)
     int nsplit;       // split streams
     int spw;          // split streams one workgroup walks, one after the other (nsplit % spw == 0)
@@ -115,7 +116,9 @@ __device__ __forceinline__ u2 deq4n(uint32_t w, h2 dd) { return deq4n2(w, dd, dd
 // fetched with a scalar load, issued one step ahead.
 __device__ __forceinline__ uint32_t lds_addr(const char * p) { return (uint32_t) (size_t) (const __attribute__((address_space(3))) char *) p; }
 __device__ __forceinline__ void dma16(const char * sbase, uint32_t voff, uint32_t lds) {
-    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "s"(lds) : "memory", "m0");
+    // (the destination is wave-uniform by construction; say so, or a value the compiler happens to keep in a vector
+    // register cannot be given to s_mov)
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" :: "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane((int) lds)) : "memory", "m0");
 }
 __device__ __forceinline__ void dma16v(const char * vaddr, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(vaddr), "s"(lds) : "memory", "m0");
@@ -140,20 +143,21 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     using C = tile_cfg<KT, D>;
     // four tile slots per wave (K and V, two each) as separate arrays, plus a small per-wave table
     __shared__ __attribute__((aligned(16))) char kb0[NWV * C::SLOT_B];
-    __shared__ __attribute__((aligned(16))) char kb1[NWV * C::SLOT_B];
     __shared__ __attribute__((aligned(16))) char vb0[NWV * C::SLOT_B];
-    __shared__ __attribute__((aligned(16))) char vb1[NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char kv1[2 * NWV * C::SLOT_B];   // K slot 1, then V slot 1
+    char * const kb1 = kv1, * const vb1 = kv1 + NWV * C::SLOT_B;
+    static_assert(32 * C::QRS <= 2 * NWV * C::SLOT_B, "the Q staging copy (at most 32 columns) fits over the second K and V slots");
     __shared__ __attribute__((aligned(16))) char tabs[NWV * C::TAB_B];
     __shared__ __attribute__((aligned(16))) char vab[NWV * C::VA_B + 16];
 
     const int lane = threadIdx.x & 63, wave = rfl(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
     // blockIdx.x -> (split stream, head group). Workgroups are dealt to the 8 XCDs round-robin by linear index, so
-    // the head groups of one split stream (which share cache lines when HPW < Hkv) are given the same index mod 8.
+    // the kv heads of one split stream (which share cache lines) are given the same index mod 8.
     // A workgroup may walk several split streams in turn (spw > 1, when a call has many more workgroups than the device
     // has CUs): stream split, split + nsplit / spw, ... - every stream is computed and written exactly as if it had a
     // workgroup of its own, only the per-workgroup set-up is shared.
-    const int HG = P.Hkv / P.HPW;
+    const int HG = P.Hkv;
     const int spw = MULTI ? P.spw : 1;
     const int nwgs = P.nsplit / spw;                          // workgroup-streams
     int split, hg;
@@ -165,10 +169,8 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         split = blockIdx.x / HG;
         hg = blockIdx.x - split * HG;
     }
-    const int hslot = wave % P.HPW;
-    const int hk = hg * P.HPW + hslot;
-    const int sub = wave / P.HPW, WPH = NWV / P.HPW;
-    const int U = 32 * WPH;                                   // positions per unit
+    const int hk = hg, sub = wave;
+    constexpr int U = 32 * NWV;                               // positions per unit
     const int row0 = blockIdx.y * P.RG;
     const int nr = min(P.RG, P.T - row0);                     // rows of this group
     const int R = nr * P.GQA;                                 // live MFMA columns
@@ -180,6 +182,8 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     char * const tab = tabs + wave * C::TAB_B;
     char * const va = vab + wave * C::VA_B;
 
+    // column -> row of the group (at most 4 rows: three comparisons instead of a division)
+    auto row_of = [&](int col) { return (col >= P.GQA) + (col >= 2 * P.GQA) + (col >= 3 * P.GQA); };
     // visible-position limit of each of this lane's columns, and the group's maximum
     int plim[NT];
     int n_max = 0, p_min = 0x7fffffff;
@@ -195,7 +199,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         const int col = 16 * r + c;
         plim[r] = -1;
         if (col < R) {
-            const int t = col / P.GQA;
+            const int t = row_of(col);
             plim[r] = P.pos_rows ? P.pos_rows[row0 + t] : p0v + row0 + t;
         }
     }
@@ -233,47 +237,63 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     };
     auto page_of = [&](int ts) -> const int32_t * { return ptab + (ts >> P.pg.psh); };
 
-    // first requests: K then V of tile 0; every later tile is requested, one load at a time, from inside the step
+    // first requests: K, then V of tile 0; every later tile is requested, one load at a time, from inside the step
     // before it, so that a wave is never parked on the memory pipeline for long while it has products to compute
-    auto first_requests = [&]() {
-    const bool have0 = tile_start(0) < n_max;
-    if (have0) {
+    size_t off0 = 0;                                          // where tile 0 starts
+    auto request_k0 = [&]() {
+        if (tile_start(0) >= n_max) return;
         int pg0 = 0;
         if (ptab) pg0 = sload_i32(page_of(tile_start(0)));
         TS(8);
         wait_scalar(pg0);
         TS(9);
-        const size_t o0 = tile_off(tile_start(0), pg0);
+        off0 = tile_off(tile_start(0), pg0);
 #pragma unroll
-        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ks0, P.kc + o0, tile_start(0), rd);
-#pragma unroll
-        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vs0, P.vc + o0, tile_start(0), rd);
-    }
+        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ks0, P.kc + off0, tile_start(0), rd);
     };
-    first_requests();
+    auto request_v0 = [&]() {
+        if (tile_start(0) >= n_max) return;
+#pragma unroll
+        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vs0, P.vc + off0, tile_start(0), rd);
+    };
+    // this wave's share of the Q rows -> LDS staging (column col at col * QRS; lane i brings floats 4 i .. 4 i + 3)
+    for (int col = wave; col < R; col += NWV) {
+        const int t = row_of(col), hh = col - t * P.GQA;
+        const float * qr = P.q + ((size_t) (row0 + t) * P.Hq + (size_t) hk * P.GQA + hh) * D;
+        if (lane < D / 4) dma16(reinterpret_cast<const char *>(qr), lane * 16, lds_addr(kv1) + col * C::QRS);
+    }
+    request_k0();
     TS(1);
 
-    // Q^T operands: column = query row (token t, head hh of the group), 8 consecutive dims per MFMA slot group
+    // Q^T operands: column = query row (token t, head hh of the group), 8 consecutive dims per MFMA slot group.
+    // The rows are the same for every wave of the workgroup: each wave has already asked for its share of them (straight
+    // into LDS, over the slots that tile 1 will use later; those requests are OLDER than the tile requests, so waiting
+    // for them does not wait for a tile), and every lane picks its operands out of that staging copy. V of tile 0 is
+    // requested only after that: while the workgroup's requests queue up at the memory pipeline a wave cannot issue
+    // anything else, so the operand set-up goes between the two halves of the queue instead of behind all of it.
+    if (tile_start(0) < n_max) wait_vm_imm<C::NRND>(); else wait_vm_imm<0>();
+    __syncthreads();
     h8 qf[NT][C::NMF];
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         const int col = 16 * r + c;
         const bool livec = col < R;
-        const int t = livec ? col / P.GQA : 0, hh = livec ? col - t * P.GQA : 0;
-        const float * qr = P.q + ((size_t) (row0 + t) * P.Hq + (size_t) hk * P.GQA + hh) * D;
+        const float * qr = reinterpret_cast<const float *>(kv1 + (livec ? col : 0) * C::QRS);
 #pragma unroll
         for (int m = 0; m < C::NMF; ++m) {
             // the 8 dims of k-slot group g of product m: f16 a run of 8; q8_0 half of a 16-code chunk; q4_0 the values
             // of nibble bytes 4 g .. 4 g + 3 of block m (low nibbles = values 4 g .., high nibbles = values 16 + 4 g ..)
             const int d0 = KT == P1A_KV_F16 ? 32 * m + 8 * g : KT == P1A_KV_Q8_0 ? 16 * (4 * (m >> 1) + g) + 8 * (m & 1) : 32 * m + 4 * g;
             const int d1 = KT == P1A_KV_Q4_0 ? d0 + 16 : d0 + 4;
-            float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-            if (livec) { a = *reinterpret_cast<const float4 *>(qr + d0); b = *reinterpret_cast<const float4 *>(qr + d1); }
+            float4 a = *reinterpret_cast<const float4 *>(qr + d0), b = *reinterpret_cast<const float4 *>(qr + d1);
+            if (!livec) a = b = make_float4(0.f, 0.f, 0.f, 0.f);
             const float s = P.qscale;
             qf[r][m] = h8{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s),
                           (half_t) (b.x * s), (half_t) (b.y * s), (half_t) (b.z * s), (half_t) (b.w * s)};
         }
     }
+    __syncthreads();                                          // the staging copy is done with: tile 1 may be requested
+    request_v0();
 
     TS(2);
     f4 o[NT][C::NDT];
@@ -284,7 +304,8 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     if (MULTI && sw) {                                                 // the next stream: the slots are free behind this barrier
         __syncthreads();
         split += nwgs;
-        first_requests();
+        request_k0();
+        request_v0();
     }
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
@@ -481,7 +502,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     }
     TS(5);
 
-    // ---- fold the WPH waves of each head (in sub order) and write one partial per (workgroup, head); the 16
+    // ---- fold the waves of the workgroup (in wave order) and write one partial per (workgroup, head); the 16
     // columns of one MFMA tile at a time, so that a column is merged the same way whatever NT is. A wave parks its
     // accumulators in its own (now idle) slots, dim quarter k in slot array k, and (m, l) in its table ----
     constexpr int QD = D / 4;                                 // dims per quarter
@@ -503,19 +524,18 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         }
         __syncthreads();
         if (r == 0) TS(6);
-        const int items = P.HPW * Rr * (D / 4);
+        const int items = Rr * (D / 4);
         for (int it = threadIdx.x; it < items; it += NWV * 64) {
-            const int d4 = it % (D / 4), rest = it / (D / 4);
-            const int cc = rest % Rr, hs = rest / Rr;
+            const int d4 = it % (D / 4), cc = it / (D / 4);
             const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
             const char * sbase = qtr == 0 ? kb0 : qtr == 1 ? kb1 : qtr == 2 ? vb0 : vb1;
             float M = NEG_INF;
-            for (int sb = 0; sb < WPH; ++sb)
-                M = fmaxf(M, reinterpret_cast<const float *>(tabs + (hs + sb * P.HPW) * C::TAB_B)[cc]);
+#pragma unroll
+            for (int w = 0; w < NWV; ++w) M = fmaxf(M, reinterpret_cast<const float *>(tabs + w * C::TAB_B)[cc]);
             f4 acc = {0.f, 0.f, 0.f, 0.f};
             float l = 0.f;
-            for (int sb = 0; sb < WPH; ++sb) {
-                const int w = hs + sb * P.HPW;
+#pragma unroll
+            for (int w = 0; w < NWV; ++w) {
                 const float * tw = reinterpret_cast<const float *>(tabs + w * C::TAB_B);
                 const float ms = tw[cc];
                 if (ms == NEG_INF) continue;
@@ -525,8 +545,8 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
                 l += tw[16 + cc] * f;
             }
             const int col = 16 * r + cc;
-            const int t = col / P.GQA, hh = col - t * P.GQA;
-            const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) (hg * P.HPW + hs) * P.GQA + hh;
+            const int t = row_of(col), hh = col - t * P.GQA;
+            const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) hg * P.GQA + hh;
             if (M != NEG_INF) *reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4) = acc;
             if (d4 == 0) {
                 float * pm = P.part_ml + (row * P.nsplit + split) * 2;
@@ -714,7 +734,7 @@ __global__ void __launch_bounds__(256) sigmoid_mul_k(float * __restrict__ x, con
 // bases and strides, pages of >= 16 positions and GQA <= 16. Everything else takes the generic kernel.
 struct dec_plan {
     bool mfma;
-    int GQA, HPW, NW, NT, RG;
+    int GQA, NW, NT, RG;
     int nsplit;    // split streams
     int NS;        // partials per output row (what merge_k folds)
     int spw;       // split streams per workgroup
@@ -739,7 +759,7 @@ dec_plan make_plan(const p1a_kv & c, int Hq, int rows_per_group, int nsplit_req,
     p.GQA = Hq / c.Hkv;
     p.mfma = mfma_ok(c, p.GQA);
     if (!p.mfma) {
-        p.HPW = 1; p.NW = 4; p.NT = 1;
+        p.NW = 4; p.NT = 1;
         p.RG = rows_per_group < 1 ? 1 : rows_per_group;   // no sharing here: the group only selects the page table
         int n = nsplit_req > 0 ? nsplit_req : 2 * cus / Hq;
         p.nsplit = n < 1 ? 1 : (n > 1024 ? 1024 : n);
@@ -748,17 +768,11 @@ dec_plan make_plan(const p1a_kv & c, int Hq, int rows_per_group, int nsplit_req,
     }
     const int cap = 32 / p.GQA < 4 ? 32 / p.GQA : 4;
     p.RG = rows_per_group < 1 ? 1 : (rows_per_group > cap ? cap : rows_per_group);
-    // tuning knobs (development A/B switches, read once): heads per workgroup and waves per workgroup
-    static const int env_hpw = env_int("P1A_DEC_HPW", 0), env_nw = env_int("P1A_DEC_NW", 0);
-    // one kv head per workgroup: its 8 waves fold into ONE partial, which keeps the split traffic at a few percent
-    // of the KV bytes; the head groups of a split stream are placed on one XCD so shared cache lines meet in its L2
-    int hpw = 1;
-    if (env_hpw > 0 && c.Hkv % env_hpw == 0 && (env_hpw == 1 || env_hpw == 2 || env_hpw == 4)) hpw = env_hpw;
-    p.HPW = hpw;
+    // One kv head per workgroup: its waves fold into ONE partial, which keeps the split traffic at a few percent of the KV
+    // bytes; the heads of a split stream are placed on one XCD so shared cache lines meet in its L2.
     const bool big_tiles = c.type == P1A_KV_F16 && c.D == 256;   // 34 KB of LDS per wave
     p.NW = big_tiles ? 4 : 8;
-    if (env_nw == 4 || (env_nw == 8 && !big_tiles)) p.NW = env_nw;
-    const int HG = c.Hkv / p.HPW;
+    const int HG = c.Hkv;
     const int wg_per_cu = p.NW == 8 ? 1 : 2;
     int n = nsplit_req > 0 ? nsplit_req : wg_per_cu * cus / HG;
     if (n >= 8) n &= ~7;
@@ -776,7 +790,7 @@ void finish_plan(dec_plan & p) {
 // 91 us at 4 - fewer, longer workgroups balance worse). The partials do not depend on it.
 int streams_per_wg(const dec_plan & p, int Hkv, int T, int cus) {
     static const int env = env_int("P1A_DEC_SPW", 0);         // development A/B knob
-    const long long wgs = (long long) p.nsplit * (Hkv / p.HPW) * ((T + p.RG - 1) / p.RG);
+    const long long wgs = (long long) p.nsplit * Hkv * ((T + p.RG - 1) / p.RG);
     const int per_round = (p.NW == 8 ? 1 : 2) * cus;
     int spw = 1;
     while (spw * 2 <= p.nsplit && p.nsplit % (spw * 2) == 0 && wgs / spw > 4LL * per_round) spw *= 2;
@@ -790,21 +804,19 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     P.q = a.q; P.kc = (const char *) c.k; P.vc = (const char *) c.v;
     P.part_o = a.part_o; P.part_ml = a.part_ml; P.pg = view_of(c);
     P.p0 = a.p0; P.p0_dev = a.p0_dev; P.pos_rows = a.pos_rows;
-    P.T = a.T; P.RG = pl.RG; P.Hq = a.Hq; P.Hkv = c.Hkv; P.GQA = pl.GQA; P.HPW = pl.HPW;
+    P.T = a.T; P.RG = pl.RG; P.Hq = a.Hq; P.Hkv = c.Hkv; P.GQA = pl.GQA;
     P.qscale = a.scale * 1.4426950408889634f; P.nsplit = pl.nsplit;
     P.spw = streams_per_wg(pl, c.Hkv, a.T, a.cus > 0 ? a.cus : 256);
-    const dim3 grid(pl.nsplit / P.spw * (c.Hkv / pl.HPW), (a.T + pl.RG - 1) / pl.RG);
+    const dim3 grid(pl.nsplit / P.spw * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
     constexpr bool big_tiles = KT == P1A_KV_F16 && D == 256;
 #define P1A_DEC(NT_, NW_) do { if (P.spw > 1) dec_mfma_k<KT, D, NT_, NW_, true><<<grid, NW_ * 64, 0, s>>>(P); \
                                else dec_mfma_k<KT, D, NT_, NW_, false><<<grid, NW_ * 64, 0, s>>>(P); } while (0)
-    if (pl.NW == 8) {
-        if constexpr (!big_tiles) {
-            if (pl.NT == 1) P1A_DEC(1, 8);
-            else P1A_DEC(2, 8);
-        }
-    } else {
+    if constexpr (big_tiles) {
         if (pl.NT == 1) P1A_DEC(1, 4);
         else P1A_DEC(2, 4);
+    } else {
+        if (pl.NT == 1) P1A_DEC(1, 8);
+        else P1A_DEC(2, 8);
     }
 #undef P1A_DEC
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
