@@ -43,7 +43,7 @@ template <uint32_t KT, int D> struct tile_cfg {
     static constexpr int SLOT_B = TILE_B > QTR_B ? TILE_B : QTR_B;   // one LDS slot
     static constexpr int VA_B = KT == P1A_KV_Q4_0 ? 16 * 144 : 0;    // q4_0: 8-byte aligned copy of a V tile's nibbles
     static constexpr int TAB_B = 256;                          // per wave: transposed V scales, later (m, l) of the merge
-    static constexpr int QRS = D * 4 + 16;                     // row stride of the Q staging copy (padded: no bank conflicts)
+    static constexpr int QRS = D * 2 + 16;                     // row stride of the f16 Q table (padded: no bank conflicts)
     static constexpr int NMF = D / 32;                         // QK MFMAs per tile
     static constexpr int NDT = D / 16;                         // output dim tiles
     static_assert(HB % 16 == 0, "head row must be a whole number of 16-byte chunks");
@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     __shared__ __attribute__((aligned(16))) char vb0[NWV * C::SLOT_B];
     __shared__ __attribute__((aligned(16))) char kv1[2 * NWV * C::SLOT_B];   // K slot 1, then V slot 1
     char * const kb1 = kv1, * const vb1 = kv1 + NWV * C::SLOT_B;
-    static_assert(32 * C::QRS <= 2 * NWV * C::SLOT_B, "the Q staging copy (at most 32 columns) fits over the second K and V slots");
+    static_assert(32 * D * 4 <= NWV * C::SLOT_B && 32 * C::QRS <= NWV * C::SLOT_B, "the Q copies (at most 32 columns) fit over the second K and V slots");
     __shared__ __attribute__((aligned(16))) char tabs[NWV * C::TAB_B];
     __shared__ __attribute__((aligned(16))) char vab[NWV * C::VA_B + 16];
 
@@ -256,44 +256,50 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 #pragma unroll
         for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vs0, P.vc + off0, tile_start(0), rd);
     };
-    // this wave's share of the Q rows -> LDS staging (column col at col * QRS; lane i brings floats 4 i .. 4 i + 3)
+    // This wave's share of the Q rows -> LDS (fp32, column col at col * 4 D bytes of K slot 1; lane i brings floats
+    // 4 i .. 4 i + 3). These requests are OLDER than the tile requests that follow, so waiting for them below does not
+    // wait for a tile.
     for (int col = wave; col < R; col += NWV) {
         const int t = row_of(col), hh = col - t * P.GQA;
         const float * qr = P.q + ((size_t) (row0 + t) * P.Hq + (size_t) hk * P.GQA + hh) * D;
-        if (lane < D / 4) dma16(reinterpret_cast<const char *>(qr), lane * 16, lds_addr(kv1) + col * C::QRS);
+        if (lane < D / 4) dma16(reinterpret_cast<const char *>(qr), lane * 16, lds_addr(kb1) + col * (D * 4));
     }
     request_k0();
+    request_v0();
     TS(1);
 
-    // Q^T operands: column = query row (token t, head hh of the group), 8 consecutive dims per MFMA slot group.
-    // The rows are the same for every wave of the workgroup: each wave has already asked for its share of them (straight
-    // into LDS, over the slots that tile 1 will use later; those requests are OLDER than the tile requests, so waiting
-    // for them does not wait for a tile), and every lane picks its operands out of that staging copy. V of tile 0 is
-    // requested only after that: while the workgroup's requests queue up at the memory pipeline a wave cannot issue
-    // anything else, so the operand set-up goes between the two halves of the queue instead of behind all of it.
-    if (tile_start(0) < n_max) wait_vm_imm<C::NRND>(); else wait_vm_imm<0>();
+    // Q^T operands: column = query row (token t, head hh of the group), 8 consecutive dims per MFMA slot group. The
+    // rows are the same for every wave of the workgroup, so the workgroup scales and rounds them once - every thread its
+    // piece - into an f16 table over V slot 1 (rows padded: conflict-free reads), and every lane picks its operands
+    // out of that. (While a workgroup's requests queue up at the memory pipeline a wave cannot issue anything else:
+    // what little work there is before the first tile is best kept short.)
+    if (tile_start(0) < n_max) wait_vm_imm<2 * C::NRND>(); else wait_vm_imm<0>();
+    __syncthreads();
+    for (int i = threadIdx.x; i < R * (D / 4); i += NWV * 64) {
+        const int col = i / (D / 4), d = 4 * (i - col * (D / 4));
+        const float4 a = *reinterpret_cast<const float4 *>(kb1 + (size_t) i * 16);
+        const float s = P.qscale;
+        *reinterpret_cast<h4 *>(vb1 + col * C::QRS + d * 2) = h4{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s)};
+    }
     __syncthreads();
     h8 qf[NT][C::NMF];
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         const int col = 16 * r + c;
         const bool livec = col < R;
-        const float * qr = reinterpret_cast<const float *>(kv1 + (livec ? col : 0) * C::QRS);
+        const char * qr = vb1 + (livec ? col : 0) * C::QRS;
 #pragma unroll
         for (int m = 0; m < C::NMF; ++m) {
             // the 8 dims of k-slot group g of product m: f16 a run of 8; q8_0 half of a 16-code chunk; q4_0 the values
             // of nibble bytes 4 g .. 4 g + 3 of block m (low nibbles = values 4 g .., high nibbles = values 16 + 4 g ..)
             const int d0 = KT == P1A_KV_F16 ? 32 * m + 8 * g : KT == P1A_KV_Q8_0 ? 16 * (4 * (m >> 1) + g) + 8 * (m & 1) : 32 * m + 4 * g;
             const int d1 = KT == P1A_KV_Q4_0 ? d0 + 16 : d0 + 4;
-            float4 a = *reinterpret_cast<const float4 *>(qr + d0), b = *reinterpret_cast<const float4 *>(qr + d1);
-            if (!livec) a = b = make_float4(0.f, 0.f, 0.f, 0.f);
-            const float s = P.qscale;
-            qf[r][m] = h8{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s),
-                          (half_t) (b.x * s), (half_t) (b.y * s), (half_t) (b.z * s), (half_t) (b.w * s)};
+            const h4 a = *reinterpret_cast<const h4 *>(qr + d0 * 2), b = *reinterpret_cast<const h4 *>(qr + d1 * 2);
+            const half_t z = (half_t) 0;
+            qf[r][m] = livec ? h8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]} : h8{z, z, z, z, z, z, z, z};
         }
     }
-    __syncthreads();                                          // the staging copy is done with: tile 1 may be requested
-    request_v0();
+    __syncthreads();                                          // both copies are done with: tile 1 may be requested
 
     TS(2);
     f4 o[NT][C::NDT];
@@ -320,6 +326,9 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         const int ts = tile_start(t);
         const int tn = tile_start(t + 1);
         const bool have_n = tn < n_max;
+        // the two waves of a SIMD take turns at the higher issue priority: the older wave would otherwise win every tie,
+        // finish its stream some 2 us before the younger one and wait for it at the fold
+        if ((t ^ (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
         int pgn = 0;
         if (ptab && have_n) pgn = sload_i32(page_of(tn));
         wait_vm_imm<C::NRND>();                               // K of tile t has landed (only its V is younger)
