@@ -278,6 +278,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload")
+    ap.add_argument("--rotating-only", action="store_true",
+                    help="skip the same-pool (Infinity Cache resident) graphs, so that every launch a profiler sees is the "
+                         "rotating-pool headline launch")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 256 MiB elementwise copy kernel (reference point for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--prefill-only", action="store_true",
@@ -327,11 +330,11 @@ def main():
     K, W = args.steps, args.warmup
     torch.cuda.synchronize()
     sec = time_graph(torch, stream, [step(i) for i in range(K)], W)
-    sec_same = time_graph(torch, stream, [step(0) for _ in range(K)], W)
+    sec_same = None if args.rotating_only else time_graph(torch, stream, [step(0) for _ in range(K)], W)
     # the dominant kernel alone (the split-K kernel; the merge kernel is switched off for this graph only)
     p1a.bench_skip_merge(True)
     sec_kernel = time_graph(torch, stream, [step(i) for i in range(K)], W)
-    sec_kernel_same = time_graph(torch, stream, [step(0) for _ in range(K)], W)
+    sec_kernel_same = None if args.rotating_only else time_graph(torch, stream, [step(0) for _ in range(K)], W)
     p1a.bench_skip_merge(False)
     gbs = step_bytes / sec / 1e9
     kgbs = step_bytes / sec_kernel / 1e9
@@ -351,22 +354,15 @@ def main():
                      "kernel_us": round(sec_kernel * 1e6, 2),
                      "note": "achieved = algorithmic KV bytes of one launch (2 * ctx * 1088 B) / average duration of the "
                              "split-K kernel, event-timed on its stream over a graph of K launches on rotating pools"},
-        "extra": {"same_pool_GBs": round(step_bytes / sec_same / 1e9, 1), "same_pool_us": round(sec_same * 1e6, 2),
-                  "kernel_same_pool_us": round(sec_kernel_same * 1e6, 2),
-                  "kernel_same_pool_GBs": round(step_bytes / sec_kernel_same / 1e9, 1),
+        "extra": {"same_pool_GBs": sec_same and round(step_bytes / sec_same / 1e9, 1), "same_pool_us": sec_same and round(sec_same * 1e6, 2),
+                  "kernel_same_pool_us": sec_kernel_same and round(sec_kernel_same * 1e6, 2),
+                  "kernel_same_pool_GBs": sec_kernel_same and round(step_bytes / sec_kernel_same / 1e9, 1),
                   "merge_kernel_us": round((sec - sec_kernel) * 1e6, 2), "nsplit": p1a.get_nsplit(Hkv)},
     }
-    # a reference point for the size: a library reduction (read-only stream) over the same number of bytes, rotating over
-    # buffers larger than the Infinity Cache - what the memory system gives a 71 MB launch that computes next to nothing
+    # a reference point for the size: a plain streaming read (nothing computed) of the same number of bytes, rotating over
+    # buffers larger than the Infinity Cache - what the memory system gives a 71 MB launch
     ref_bufs = [torch.ones(step_bytes // 4, device="cuda") for _ in range(n_pools)]
-    ref_out = torch.empty((), device="cuda")
-    it_ref = [0]
-
-    def ref_step():   # (eager, not captured: the library's reduction clears its own scratch memory)
-        it_ref[0] += 1
-        torch.sum(ref_bufs[it_ref[0] % n_pools], dim=0, out=ref_out)
-
-    sec_ref = time_eager(torch, ref_step, reps=64, warmup=8)
+    sec_ref = time_graph(torch, stream, [(lambda i=i: p1a.bench_stream_read(ref_bufs[i % n_pools])) for i in range(min(K, 64))], W)
     res["extra"]["stream_read_same_bytes_us"] = round(sec_ref * 1e6, 2)
     res["extra"]["stream_read_same_bytes_GBs"] = round(step_bytes / sec_ref / 1e9, 1)
     del ref_bufs

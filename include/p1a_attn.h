@@ -175,6 +175,10 @@ void p1a_set_nsplit(int n);
 /* Benchmarks only (no counterpart in the reference, whose benches time both kernels together): when on,
  * p1a_attn_decode stops after the split-K kernel and leaves `out` untouched, so that kernel can be event-timed alone. */
 void p1a_bench_skip_merge(int on);
+/* Benchmarks only (no counterpart in the reference): a plain read of `bytes` bytes of device memory (16 bytes per lane,
+ * one contiguous span per workgroup, nothing computed) - the time the memory system needs for a launch of that size,
+ * to set a decode launch of the same number of KV bytes against. bytes is rounded down to a multiple of 16. */
+int p1a_bench_stream_read(const void *src, size_t bytes, void *stream);
 /* free every scratch buffer of the current process (after synchronising the devices that own them) */
 void p1a_release(void);
 

@@ -8,7 +8,7 @@ KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
     "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
-    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_release", "p1a_last_error",
+    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
     "p1a_version",
     # include/p1a_pool.h
     "p1a_pool_create", "p1a_pool_destroy", "p1a_pool_n_pages", "p1a_pool_free_pages", "p1a_pool_max_pages", "p1a_pool_page_bytes",
@@ -89,6 +89,8 @@ def lib():
     L.p1a_set_nsplit.argtypes = [i32]
     L.p1a_bench_skip_merge.restype = None
     L.p1a_bench_skip_merge.argtypes = [i32]
+    L.p1a_bench_stream_read.restype = i32
+    L.p1a_bench_stream_read.argtypes = [vp, sz, vp]
     L.p1a_release.restype = None
     L.p1a_last_error.restype = ctypes.c_char_p
     L.p1a_version.restype = ctypes.c_char_p
@@ -305,6 +307,11 @@ def set_nsplit(n):
 
 def bench_skip_merge(on):
     lib().p1a_bench_skip_merge(1 if on else 0)
+
+
+def bench_stream_read(t):
+    """Benchmarks only: a plain streaming read of the tensor's bytes on the current stream."""
+    _check(lib().p1a_bench_stream_read(_ptr(t), t.numel() * t.element_size(), _stream()), "p1a_bench_stream_read")
 
 
 class KVDesc:

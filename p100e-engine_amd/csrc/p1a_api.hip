@@ -239,6 +239,11 @@ void p1a_set_nsplit(int n) { g_nsplit_override = n > 0 ? n : 0; }
 
 void p1a_bench_skip_merge(int on) { g_skip_merge = on != 0; }
 
+int p1a_bench_stream_read(const void * src, size_t bytes, void * stream) {
+    if (!src || bytes < 16 || ((uintptr_t) src & 15)) { set_error("p1a_bench_stream_read: null, short or misaligned source"); return P1A_E_ARG; }
+    return launch_stream_read(src, bytes, (hipStream_t) stream);
+}
+
 void p1a_release(void) {
     std::lock_guard<std::mutex> lk(g_mu);
     int cur = 0;

@@ -110,6 +110,7 @@ int launch_ew_quant(int op, const float * a, const float * b, float * y, void * 
 int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s);
 int launch_sigmoid_mul(float * x, const float * g, size_t n, hipStream_t s);
+int launch_stream_read(const void * src, size_t bytes, hipStream_t s);   // benchmarks only
 
 void set_error(const char * fmt, ...);
 

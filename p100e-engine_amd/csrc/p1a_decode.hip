@@ -880,6 +880,32 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
 extern "C" void p1a_set_trace(long long * buf) { (void) hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &buf, sizeof buf); }
 #endif
 
+// Benchmarks only: a plain streaming read. Workgroup b reads one contiguous span, every lane 16 bytes at a time with four
+// loads in flight; the sum is kept so that the loads cannot be dropped, and stored nowhere (it never equals the sentinel
+// for the inputs a benchmark uses; one float of static device memory takes it if it ever does).
+__device__ float g_stream_read_sink;
+__global__ void __launch_bounds__(512) stream_read_k(const f4 * __restrict__ p, size_t n16) {
+    const size_t per = n16 / gridDim.x;
+    const f4 * b = p + per * blockIdx.x;
+    const size_t n = blockIdx.x + 1 == gridDim.x ? n16 - per * blockIdx.x : per;
+    f4 acc = {0.f, 0.f, 0.f, 0.f};
+    size_t i = threadIdx.x;
+    for (; i + 3 * 512 < n; i += 4 * 512) {
+        const f4 v0 = __builtin_nontemporal_load(b + i), v1 = __builtin_nontemporal_load(b + i + 512);
+        const f4 v2 = __builtin_nontemporal_load(b + i + 1024), v3 = __builtin_nontemporal_load(b + i + 1536);
+        acc += (v0 + v1) + (v2 + v3);
+    }
+    for (; i < n; i += 512) acc += __builtin_nontemporal_load(b + i);
+    if (acc[0] + acc[1] + acc[2] + acc[3] == -1.2345678e38f) g_stream_read_sink = acc[0];
+}
+
+int launch_stream_read(const void * src, size_t bytes, hipStream_t s) {
+    int dev = 0, cus = 256;
+    if (hipGetDevice(&dev) == hipSuccess) (void) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    stream_read_k<<<cus > 0 ? cus : 256, 512, 0, s>>>(reinterpret_cast<const f4 *>(src), bytes / 16);
+    return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
+}
+
 int launch_sigmoid_mul(float * x, const float * g, size_t n, hipStream_t s) {
     const size_t nb = (n + 255) / 256;
     sigmoid_mul_k<<<(unsigned) (nb > 4096 ? 4096 : (nb ? nb : 1)), 256, 0, s>>>(x, g, n);
