@@ -141,6 +141,28 @@ def test_config4_verify_blocks(p1a, kv_type):
     check(out.cpu().numpy(), ref, "config 4 (reduced)")
 
 
+@pytest.mark.parametrize("kv_type,Hq,Hkv,rows", [(O.KV_Q8_0, 16, 2, 4), (O.KV_Q4_0, 32, 2, 2), (O.KV_F16, 16, 2, 4), (O.KV_Q8_0, 14, 2, 4)])
+def test_widest_row_groups(p1a, kv_type, Hq, Hkv, rows):
+    """Row groups that fill both 16-column tiles (GQA 8 x 4 rows, GQA 16 x 2 rows: 32 live columns, the most the
+    workgroup's Q table holds) and one that leaves the second tile ragged (GQA 7 x 4 rows = 28): each row vs the oracle,
+    and bit for bit the row of a call of its own"""
+    D, psh, n = 256, 6, 1500
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n, n], seed=61)
+    T = 2 * rows
+    q, _, _, gate = I.qkv(62, 1, T, Hq, Hkv, D)
+    pos = np.array([n - rows + t for _ in range(2) for t in range(rows)], np.int32)
+    rtab = np.array([s * pool.maxp for s in range(2) for _ in range(rows)], np.int32)
+    ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, 1 / 16, gate=gate)
+    out = torch.empty((T, Hq, D), device="cuda")
+    p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, T, dev(pos), Hq, 1 / 16, gate=dev(gate), rows_per_seq=rows)
+    check(out.cpu().numpy(), ref, f"row groups of {rows} x GQA {Hq // Hkv}")
+    for t in range(T):
+        one = torch.empty((1, Hq, D), device="cuda")
+        p1a.attn_decode_rows(dev(q[t:t + 1]), pool.devkv.with_rows(dev(rtab[t:t + 1])), one, 1, dev(pos[t:t + 1]), Hq, 1 / 16,
+                             gate=dev(gate[t:t + 1]))
+        assert torch.equal(one[0], out[t]), t
+
+
 def test_other_shapes_and_refusals(p1a):
     # GQA 4 / D 128 f16, GQA 8 / D 64 f16 (MFMA path), q8_0 at D 128 (generic path)
     for kv_type, Hq, Hkv, D in [(O.KV_F16, 8, 2, 128), (O.KV_F16, 8, 1, 64), (O.KV_Q8_0, 8, 2, 128), (O.KV_Q4_0, 6, 3, 96)]:
