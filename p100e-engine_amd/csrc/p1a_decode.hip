@@ -1,20 +1,21 @@
 // Split-K paged-KV decode / MTP-verify attention for gfx950 (MI355X).
 //
 // Work decomposition
-//   grid = (nsplit * head groups, row groups), block = NW waves (8, or 4 when a tile is large). A row group is up to
-//   4 query rows of ONE sequence (the tokens of a verify block); its GQA * rows query rows are the columns of 16-wide
+//   grid = (nsplit * kv heads, row groups), block = NW waves (8, or 4 when a tile is large). A row group is up to 4
+//   query rows of ONE sequence (the tokens of a verify block); its GQA * rows query rows are the columns of 16-wide
 //   MFMA tiles, so the group's KV is read once. A workgroup owns one kv head; in unit u (32 * NW positions) wave w owns
-//   the 32 consecutive positions 32 w .., which it walks as two
-//   16-key tiles; split stream s owns the units s, s + nsplit, ... . The partition depends only on the device and
-//   Hkv, never on T, the depth or the batch, so a row is computed by the same sequence of operations whichever call
-//   it is part of (T-invariance, rows == single, paged == contiguous).
+//   the 32 consecutive positions 32 w .., which it walks as two 16-key tiles; split stream s owns the units s,
+//   s + nsplit, ... . The partition depends only on the device and Hkv, never on T, the depth or the batch, so a row
+//   is computed by the same sequence of operations whichever call it is part of (T-invariance, rows == single,
+//   paged == contiguous).
 // Data movement
 //   A 16-key tile of one head (K or V) is fetched by global_load_lds_dwordx4: 16 bytes per lane in memory order (17
 //   consecutive lanes cover one q8_0 head row), written by the memory pipeline straight into a wave-private LDS slot
 //   that is the linear image of those rows - no staging registers, no workgroup barrier in the key loop. K and V have
-//   two slots each; the tile two steps ahead is requested as soon as a slot has been consumed, so every wave keeps
-//   about three tiles in flight while it computes. Each slot is its own __shared__ array so that the compiler can
-//   tell which outstanding load a given LDS read depends on and wait for exactly that one.
+//   two slots each; the loads of tile t + 1 are issued between the products of tile t, and the in-order vector-memory
+//   counter tells which tile has landed. The Q rows are the same for all waves of a workgroup: they are requested
+//   first (older than every tile request), once, straight into LDS, and scaled and rounded into an f16 table that the
+//   lanes pick their MFMA operands from.
 // Arithmetic
 //   S^T = K Q^T on v_mfma_f32_16x16x32_f16 and O^T = V^T P^T on v_mfma_f32_16x16x16_f16: q8_0 codes are expanded to
 //   f16 in registers with a byte-permute (0x6400 | code ^ 0x80 = 1152 + code) and multiplied by the f16 block scale;
@@ -141,7 +142,7 @@ __device__ __forceinline__ void wait_scalar(int & v) { asm volatile("s_waitcnt l
 template <uint32_t KT, int D, int NT, int NWV, bool MULTI>
 __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
-    // four tile slots per wave (K and V, two each) as separate arrays, plus a small per-wave table
+    // four tile slots per wave (K and V, two each), plus a small per-wave table
     __shared__ __attribute__((aligned(16))) char kb0[NWV * C::SLOT_B];
     __shared__ __attribute__((aligned(16))) char vb0[NWV * C::SLOT_B];
     __shared__ __attribute__((aligned(16))) char kv1[2 * NWV * C::SLOT_B];   // K slot 1, then V slot 1
@@ -538,20 +539,27 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             const int d4 = it % (D / 4), cc = it / (D / 4);
             const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
             const char * sbase = qtr == 0 ? kb0 : qtr == 1 ? kb1 : qtr == 2 ? vb0 : vb1;
+            // every LDS read first (they do not depend on one another), then the arithmetic; a wave that saw no visible
+            // key (m = -inf) parked zeros and gets the factor 0
+            float mw[NWV], lw[NWV];
+            f4 aw[NWV];
+#pragma unroll
+            for (int w = 0; w < NWV; ++w) {
+                const float * tw = reinterpret_cast<const float *>(tabs + w * C::TAB_B);
+                mw[w] = tw[cc];
+                lw[w] = tw[16 + cc];
+                aw[w] = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * QD + dq);
+            }
             float M = NEG_INF;
 #pragma unroll
-            for (int w = 0; w < NWV; ++w) M = fmaxf(M, reinterpret_cast<const float *>(tabs + w * C::TAB_B)[cc]);
+            for (int w = 0; w < NWV; ++w) M = fmaxf(M, mw[w]);
             f4 acc = {0.f, 0.f, 0.f, 0.f};
             float l = 0.f;
 #pragma unroll
             for (int w = 0; w < NWV; ++w) {
-                const float * tw = reinterpret_cast<const float *>(tabs + w * C::TAB_B);
-                const float ms = tw[cc];
-                if (ms == NEG_INF) continue;
-                const float f = __builtin_amdgcn_exp2f(ms - M);
-                const f4 a = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * QD + dq);
-                acc += a * f;
-                l += tw[16 + cc] * f;
+                const float f = mw[w] == NEG_INF ? 0.f : __builtin_amdgcn_exp2f(mw[w] - M);
+                acc += aw[w] * f;
+                l += lw[w] * f;
             }
             const int col = 16 * r + cc;
             const int t = row_of(col), hh = col - t * P.GQA;
