@@ -679,11 +679,10 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
     // the gate depends on nothing here: its load rides along with the first batch of partials
     f4 gt = {0.f, 0.f, 0.f, 0.f};
     if (gate && sl == 0) gt = *reinterpret_cast<const f4 *>(gate + row * D + d);
-    float M = NEG_INF;
-    for (int s = tid; s < NS; s += 64) M = fmaxf(M, ml[2 * s]);
-    // the partials do not depend on M: request the first batch before the maximum is reduced
+    // the first batch of partials (all of them when NS <= 64) is requested before anything is known about the maximum
     f4 a[CH];
     float ms[CH], ls[CH];
+    float M = NEG_INF;
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
         const int s = sl + 8 * k;
@@ -693,8 +692,13 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
             a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS + s) * D + d);
         }
     }
+    // the maximum over all splits: this slice's (its first batch is in registers already; later batches re-read the pairs),
+    // then over the 8 slices - the lanes that share (lane & 7)
+    for (int s = sl + 8 * CH; s < NS; s += 8) M = fmaxf(M, ml[2 * s]);
 #pragma unroll
-    for (int w = 32; w > 0; w >>= 1) M = fmaxf(M, __shfl_xor(M, w));
+    for (int k = 0; k < CH; ++k) M = fmaxf(M, ms[k]);
+    M = fmaxf(M, __shfl_xor(M, 8));
+    M = max_over_groups(M);
     f4 num = {0.f, 0.f, 0.f, 0.f};
     float den = 0.f;
     for (int s0 = sl; s0 < NS; s0 += 8 * CH) {
