@@ -72,6 +72,8 @@ struct dec_params {
     float qscale;     // softmax scale * log2(e)
     int nsplit;       // split streams
     int spw;          // split streams one workgroup walks, one after the other (nsplit % spw == 0)
+    int hkv_sh;       // log2(Hkv) when Hkv is a power of two, else -1
+    int npt;          // page-table entries of one sequence (ceil(n_ctx / page positions)); 0 = contiguous
 };
 
 __device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
@@ -164,8 +166,9 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     int split, hg;
     if ((nwgs & 7) == 0) {
         const int i = blockIdx.x, j = i >> 3;
-        hg = j % HG;
-        split = (j / HG) * 8 + (i & 7);
+        const int jq = P.hkv_sh >= 0 ? j >> P.hkv_sh : j / HG;
+        hg = j - jq * HG;
+        split = jq * 8 + (i & 7);
     } else {
         split = blockIdx.x / HG;
         hg = blockIdx.x - split * HG;
@@ -175,6 +178,11 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     const int row0 = blockIdx.y * P.RG;
     const int nr = min(P.RG, P.T - row0);                     // rows of this group
     const int R = nr * P.GQA;                                 // live MFMA columns
+    // the page-table entry of this wave's first tile is asked for before anything else (it is the first link of the
+    // chain entry -> tile address -> tile); the index is clamped into the table, the entry is only used if the tile exists
+    const int32_t * ptab = kv_tab(P.pg, P.pos_rows ? row0 : 0);
+    int pg0_early = 0;
+    if (ptab) pg0_early = sload_i32(ptab + min((split * U + sub * 32) >> P.pg.psh, P.npt - 1));
     const int p0v = P.pos_rows ? 0 : (P.p0_dev ? *P.p0_dev : P.p0);
     TS(0);
 
@@ -204,7 +212,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             plim[r] = P.pos_rows ? P.pos_rows[row0 + t] : p0v + row0 + t;
         }
     }
-    const int32_t * ptab = kv_tab(P.pg, P.pos_rows ? row0 : 0);
     const size_t head_off = (size_t) hk * C::HB;
     const int rowb = (int) P.pg.rowb;
 
@@ -241,10 +248,10 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     // first requests: K, then V of tile 0; every later tile is requested, one load at a time, from inside the step
     // before it, so that a wave is never parked on the memory pipeline for long while it has products to compute
     size_t off0 = 0;                                          // where tile 0 starts
-    auto request_k0 = [&]() {
+    auto request_k0 = [&](bool first) {
         if (tile_start(0) >= n_max) return;
-        int pg0 = 0;
-        if (ptab) pg0 = sload_i32(page_of(tile_start(0)));
+        int pg0 = pg0_early;
+        if (ptab && !first) pg0 = sload_i32(page_of(tile_start(0)));
         TS(8);
         wait_scalar(pg0);
         TS(9);
@@ -265,7 +272,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         const float * qr = P.q + ((size_t) (row0 + t) * P.Hq + (size_t) hk * P.GQA + hh) * D;
         if (lane < D / 4) dma16(reinterpret_cast<const char *>(qr), lane * 16, lds_addr(kb1) + col * (D * 4));
     }
-    request_k0();
+    request_k0(true);
     request_v0();
     TS(1);
 
@@ -311,7 +318,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     if (MULTI && sw) {                                                 // the next stream: the slots are free behind this barrier
         __syncthreads();
         split += nwgs;
-        request_k0();
+        request_k0(false);
         request_v0();
     }
 #pragma unroll
@@ -828,6 +835,9 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     P.T = a.T; P.RG = pl.RG; P.Hq = a.Hq; P.Hkv = c.Hkv; P.GQA = pl.GQA;
     P.qscale = a.scale * 1.4426950408889634f; P.nsplit = pl.nsplit;
     P.spw = streams_per_wg(pl, c.Hkv, a.T, a.cus > 0 ? a.cus : 256);
+    P.hkv_sh = -1;
+    for (int sh = 0; sh < 16; ++sh) if ((1 << sh) == c.Hkv) P.hkv_sh = sh;
+    P.npt = c.pt ? (int) (((long long) c.n_ctx + (1LL << c.psh) - 1) >> c.psh) : 0;
     const dim3 grid(pl.nsplit / P.spw * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
     constexpr bool big_tiles = KT == P1A_KV_F16 && D == 256;
 #define P1A_DEC(NT_, NW_) do { if (P.spw > 1) dec_mfma_k<KT, D, NT_, NW_, true><<<grid, NW_ * 64, 0, s>>>(P); \
