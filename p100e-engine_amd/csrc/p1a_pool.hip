@@ -128,18 +128,27 @@ int restore_impl(p1a_pool * p, int id, int np, bool state) {
     q->slot = p->free_slots.back();
     p->free_slots.pop_back();
     q->pages.clear();
+    // a failure below leaves the sequence as it was: offloaded, its host copy intact, pages and slot given back
+    auto undo = [&](int rc) {
+        (void) p->sync();
+        for (auto it = q->pages.rbegin(); it != q->pages.rend(); ++it) p->free_pages.push_back(*it);
+        q->pages.clear();
+        p->free_slots.push_back(q->slot);
+        q->slot = -1;
+        return rc;
+    };
     if (np > 0) {
         const int rc = p1a_seq_ensure_pages(p, id, std::min(np << p->cfg.psh, p->cfg.n_ctx));
-        if (rc < 0) return rc;
+        if (rc < 0) return undo(rc);
     }
     for (int i = 0; i < np; ++i)
-        if (!image_to_page(p, q->host + (size_t) i * p->page_bytes, q->pages[i], hipMemcpyHostToDevice)) return P1A_E_LAUNCH;
+        if (!image_to_page(p, q->host + (size_t) i * p->page_bytes, q->pages[i], hipMemcpyHostToDevice)) return undo(P1A_E_LAUNCH);
     const char * st = q->host + (size_t) q->host_pages * p->page_bytes;
     if (p->cfg.state_bytes) {
-        if (state) { if (!p->copy(p->state_of(q->slot), st, p->cfg.state_bytes, hipMemcpyHostToDevice)) return P1A_E_LAUNCH; }
-        else if (!p->zero(p->state_of(q->slot), p->cfg.state_bytes)) return P1A_E_LAUNCH;
+        if (state) { if (!p->copy(p->state_of(q->slot), st, p->cfg.state_bytes, hipMemcpyHostToDevice)) return undo(P1A_E_LAUNCH); }
+        else if (!p->zero(p->state_of(q->slot), p->cfg.state_bytes)) return undo(P1A_E_LAUNCH);
     }
-    if (!p->sync()) return P1A_E_LAUNCH;
+    if (!p->sync()) return undo(P1A_E_LAUNCH);
     p->pin_free(q->host);
     q->host = nullptr;
     p->host_bytes -= q->host_bytes;
@@ -283,7 +292,11 @@ int p1a_seq_create(p1a_pool * p) {
     q.used = true;
     q.slot = p->free_slots.back();
     p->free_slots.pop_back();
-    if (!p->zero(p->state_of(q.slot), p->cfg.state_bytes)) return P1A_E_LAUNCH;
+    if (!p->zero(p->state_of(q.slot), p->cfg.state_bytes)) {
+        p->free_slots.push_back(q.slot);
+        q = seq_t{};
+        return P1A_E_LAUNCH;
+    }
     return id;
 }
 
@@ -381,16 +394,17 @@ int p1a_seq_fork(p1a_pool * p, int src, int n) {
     const int id = p1a_seq_create(p);   // may grow the sequence table: pointers taken after
     if (id < 0) return id;
     const int np = p->pages_for(n);
+    auto drop = [&](int rc) { (void) p1a_seq_free(p, id); return rc; };   // a failed fork leaves no half-made copy behind
     if (np > 0) {
         const int rc = p1a_seq_ensure_pages(p, id, std::min(np << p->cfg.psh, p->cfg.n_ctx));
-        if (rc < 0) return rc;
+        if (rc < 0) return drop(rc);
     }
     const seq_t & q = p->seqs[src];
     seq_t & d = p->seqs[id];
     for (int i = 0; i < np; ++i)   // every KV layer's K and V of page i: one 2-D copy (rows = 2 x layers, pitch = a region)
         if (!p->copy2d(p->kv_pool + (size_t) d.pages[i] * p->pblk, p->region(), p->kv_pool + (size_t) q.pages[i] * p->pblk,
-                       p->region(), p->pblk, (size_t) 2 * p->cfg.n_kv_layers, hipMemcpyDeviceToDevice)) return P1A_E_LAUNCH;
-    if (!p->sync()) return P1A_E_LAUNCH;
+                       p->region(), p->pblk, (size_t) 2 * p->cfg.n_kv_layers, hipMemcpyDeviceToDevice)) return drop(P1A_E_LAUNCH);
+    if (!p->sync()) return drop(P1A_E_LAUNCH);
     d.n_past = n;
     d.toks.assign(q.toks.begin(), q.toks.begin() + n);
     return id;
@@ -407,10 +421,11 @@ int p1a_seq_offload(p1a_pool * p, int id) {
     if (!p->sync()) return P1A_E_LAUNCH;
     q->host = p->pin_alloc(bytes);
     if (!q->host) { set_error("seq_offload: pinned host allocation of %zu MiB failed", bytes >> 20); return P1A_E_SCRATCH; }
+    auto undo = [&](int rc) { (void) p->sync(); p->pin_free(q->host); q->host = nullptr; return rc; };   // still resident
     for (size_t i = 0; i < q->pages.size(); ++i)
-        if (!page_to_image(p, q->pages[i], q->host + i * p->page_bytes, hipMemcpyDeviceToHost)) return P1A_E_LAUNCH;
-    if (!p->copy(q->host + q->pages.size() * p->page_bytes, p->state_of(q->slot), p->cfg.state_bytes, hipMemcpyDeviceToHost)) return P1A_E_LAUNCH;
-    if (!p->sync()) return P1A_E_LAUNCH;
+        if (!page_to_image(p, q->pages[i], q->host + i * p->page_bytes, hipMemcpyDeviceToHost)) return undo(P1A_E_LAUNCH);
+    if (!p->copy(q->host + q->pages.size() * p->page_bytes, p->state_of(q->slot), p->cfg.state_bytes, hipMemcpyDeviceToHost)) return undo(P1A_E_LAUNCH);
+    if (!p->sync()) return undo(P1A_E_LAUNCH);
     q->host_pages = (int) q->pages.size();
     q->host_bytes = bytes;
     p->host_bytes += bytes;
