@@ -104,6 +104,38 @@ def test_bitwise_invariances(p1a, kv_type):
         assert torch.equal(one[0], out[t]), ("blocks", t)
 
 
+@pytest.mark.parametrize("kv_type", [O.KV_F16, O.KV_Q8_0])
+def test_t_invariance_sweep(p1a, kv_type):
+    """Row t of a T-row call == the T = 1 call at p0 + t, bit for bit, at every depth 0..300 and every 37th up to 4096
+    (the sweep of the reference's tests/fast_tinv_test.cu:41-60: Hq 12 / Hkv 2), and device p0 == host p0"""
+    Hq, Hkv, D, psh, n = 12, 2, 256, 6, 4100
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n], seed=15, fill="device")
+    k = I.normal(I.rng(16), (n, Hkv, D))
+    v = I.normal(I.rng(17), (n, Hkv, D))
+    c = pool.dev_seq(0)
+    p1a.kv_append(c, dev(k), dev(v), 0, n)
+    dq = dev(I.normal(I.rng(18), (4, Hq, D)))
+    depths = list(range(0, 301)) + list(range(300, 4096, 37))
+    singles = {}
+    one = torch.empty((1, Hq, D), device="cuda")
+    p0d = dev(np.array([0], np.int32))
+    for p0 in depths:
+        for T in (2, 3, 4):
+            a = torch.empty((T, Hq, D), device="cuda")
+            p1a.attn_decode(dq, c, a, T, p0, Hq, 1 / 16)
+            if T == 4:
+                b = torch.empty((T, Hq, D), device="cuda")
+                p0d.fill_(p0)
+                p1a.attn_decode_dev(dq, c, b, T, p0d, n, Hq, 1 / 16)
+                assert torch.equal(a, b), ("device p0", p0)
+            for t in range(T):
+                key = (t, p0 + t)
+                if key not in singles:
+                    p1a.attn_decode(dq[t:t + 1], c, one, 1, p0 + t, Hq, 1 / 16)
+                    singles[key] = one[0].clone()
+                assert torch.equal(singles[key], a[t]), (T, p0, t)
+
+
 def test_config3_batched_slots(p1a):
     """8 slots sharing one paged q8_0 pool, lengths log-uniform in [1024, 32768] (scaled down 8x here; test_gpu_full_size.py runs the full size), page tables interleaved, one row per slot"""
     Hq, Hkv, D, psh = 24, 4, 256, 8
