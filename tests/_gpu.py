@@ -69,4 +69,5 @@ def check(out, ref, what=""):
     ma, rl = I.errors(out, ref)
     assert np.all(np.isfinite(out)), what
     assert ma <= I.MAX_ABS_TOL and rl <= I.REL_L2_TOL, f"{what}: max_abs={ma:.3e} rel_l2={rl:.3e}"
+    print(f"[parity] {what}: max_abs={ma:.3e} (tol {I.MAX_ABS_TOL:g}) rel_l2={rl:.3e} (tol {I.REL_L2_TOL:g})")   # shown with pytest -s
     return ma, rl
