@@ -181,8 +181,11 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     // the page-table entry of this wave's first tile is asked for before anything else (it is the first link of the
     // chain entry -> tile address -> tile); the index is clamped into the table, the entry is only used if the tile exists
     const int32_t * ptab = kv_tab(P.pg, P.pos_rows ? row0 : 0);
+    // (n_ctx only bounds the read here: an entry fetched through a clamped index is fetched again, unclamped, once the
+    // tile is known to exist)
+    const int idx_early = max(0, min((split * U + sub * 32) >> P.pg.psh, P.npt - 1));
     int pg0_early = 0;
-    if (ptab) pg0_early = sload_i32(ptab + min((split * U + sub * 32) >> P.pg.psh, P.npt - 1));
+    if (ptab) pg0_early = sload_i32(ptab + idx_early);
     const int p0v = P.pos_rows ? 0 : (P.p0_dev ? *P.p0_dev : P.p0);
     TS(0);
 
@@ -251,7 +254,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     auto request_k0 = [&](bool first) {
         if (tile_start(0) >= n_max) return;
         int pg0 = pg0_early;
-        if (ptab && !first) pg0 = sload_i32(page_of(tile_start(0)));
+        if (ptab && (!first || (tile_start(0) >> P.pg.psh) != idx_early)) pg0 = sload_i32(page_of(tile_start(0)));
         TS(8);
         wait_scalar(pg0);
         TS(9);

@@ -195,6 +195,22 @@ def test_widest_row_groups(p1a, kv_type, Hq, Hkv, rows):
         assert torch.equal(one[0], out[t]), t
 
 
+def test_descriptor_n_ctx_only_bounds(p1a):
+    """n_ctx of the descriptor is the caller's word; the kernel uses it to bound an early page-table read, never to pick a
+    page: an understated (or missing) n_ctx gives the same bits"""
+    Hq, Hkv, D, psh, n = 24, 4, 256, 5, 3000
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, psh, [n], seed=71)
+    dq = dev(I.normal(I.rng(72), (2, Hq, D)))
+    c = pool.dev_seq(0)
+    ref = torch.empty((2, Hq, D), device="cuda")
+    p1a.attn_decode(dq, c, ref, 2, n - 2, Hq, 1 / 16)
+    for n_ctx in (0, 1, 64, 1000):
+        c.n_ctx = n_ctx
+        out = torch.empty((2, Hq, D), device="cuda")
+        p1a.attn_decode(dq, c, out, 2, n - 2, Hq, 1 / 16)
+        assert torch.equal(out, ref), n_ctx
+
+
 def test_other_shapes_and_refusals(p1a):
     # GQA 4 / D 128 f16, GQA 8 / D 64 f16 (MFMA path), q8_0 at D 128 (generic path)
     for kv_type, Hq, Hkv, D in [(O.KV_F16, 8, 2, 128), (O.KV_F16, 8, 1, 64), (O.KV_Q8_0, 8, 2, 128), (O.KV_Q4_0, 6, 3, 96)]:
