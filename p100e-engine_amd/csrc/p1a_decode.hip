@@ -40,7 +40,9 @@ template <uint32_t KT, int D> struct tile_cfg {
     static constexpr int NCH = 16 * CPK;                       // chunks per 16-key tile
     static constexpr int NRND = (NCH + 63) / 64;               // load rounds per tile
     static constexpr int TILE_B = 16 * HB;                     // the linear image of 16 head rows
-    static constexpr int QTR_B = 16 * (D / 4) * 4;             // one dim quarter of a wave's accumulators (merge epilogue)
+    static constexpr int QDP = D / 4 + 4;                      // floats per column of a parked dim quarter: padded, or the 16
+                                                               // columns of a store would all start in the same LDS bank
+    static constexpr int QTR_B = 16 * QDP * 4;                 // one dim quarter of a wave's accumulators (merge epilogue)
     static constexpr int SLOT_B = TILE_B > QTR_B ? TILE_B : QTR_B;   // one LDS slot
     static constexpr int VA_B = KT == P1A_KV_Q4_0 ? 16 * 144 : 0;    // q4_0: 8-byte aligned copy of a V tile's nibbles
     static constexpr int TAB_B = 256;                          // per wave: transposed V scales, later (m, l) of the merge
@@ -535,7 +537,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 #pragma unroll
             for (int j = 0; j < C::NDT; ++j) {
                 float * dst = reinterpret_cast<float *>(st[j / (C::NDT / 4)] + wave * C::SLOT_B);
-                *reinterpret_cast<f4 *>(dst + c * QD + 16 * (j % (C::NDT / 4)) + 4 * g) = o[r][j];
+                *reinterpret_cast<f4 *>(dst + c * C::QDP + 16 * (j % (C::NDT / 4)) + 4 * g) = o[r][j];
             }
             if (g == 0) {
                 reinterpret_cast<float *>(tab)[c] = m_run[r];
@@ -558,7 +560,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
                 const float * tw = reinterpret_cast<const float *>(tabs + w * C::TAB_B);
                 mw[w] = tw[cc];
                 lw[w] = tw[16 + cc];
-                aw[w] = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * QD + dq);
+                aw[w] = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * C::QDP + dq);
             }
             float M = NEG_INF;
 #pragma unroll
