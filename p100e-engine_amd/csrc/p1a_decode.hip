@@ -365,9 +365,15 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         } else if constexpr (KT == P1A_KV_Q4_0) {   // 8 blocks of 18 B: f16 scale, then 16 nibble bytes (2-byte aligned)
 #pragma unroll
             for (int b = 0; b < C::NMF; ++b) {
-                const uint16_t * blk = reinterpret_cast<const uint16_t *>(krow + 18 * b);
-                const uint32_t d16 = blk[0];
-                const uint32_t w = (uint32_t) blk[1 + 2 * g] | ((uint32_t) blk[2 + 2 * g] << 16);   // nibble bytes 4 g .. 4 g + 3
+                // nibble bytes 4 g .. 4 g + 3 of block b sit at 18 b + 2 + 4 g: a whole dword in odd blocks, the upper and
+                // lower halves of two neighbouring dwords in even ones (head rows start 16-byte aligned)
+                const uint32_t d16 = *reinterpret_cast<const uint16_t *>(krow + 18 * b);
+                uint32_t w;
+                if (b & 1) w = *reinterpret_cast<const uint32_t *>(krow + 18 * b + 2 + 4 * g);   // (b is a constant once unrolled)
+                else {
+                    const uint32_t * pw = reinterpret_cast<const uint32_t *>(krow + 18 * b + 4 * g);
+                    w = __builtin_amdgcn_alignbit(pw[1], pw[0], 16);
+                }
                 const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
                 const u2 lo = deq4n(w & 0x0f0f0f0fu, dd), hi = deq4n((w >> 4) & 0x0f0f0f0fu, dd);
                 const u4 a = {lo.lo, lo.hi, hi.lo, hi.hi};
@@ -453,14 +459,23 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             {   // re-align: nibble bytes of block bb of a key -> va[key][bb][16] (8-byte aligned for the transposing read);
                 // scales -> tab[block][key]
                 const int key = lane & 15, q2 = lane >> 4;
-#pragma unroll
-                for (int x = 0; x < 2; ++x) {
-                    const int bb = 2 * q2 + x;
-                    const uint16_t * blk = reinterpret_cast<const uint16_t *>(vs + key * C::HB + 18 * bb);
-                    *reinterpret_cast<uint16_t *>(tab + bb * 32 + key * 2) = blk[0];
-                    u4 n;
-#pragma unroll
-                    for (int k = 0; k < 4; ++k) n[k] = (uint32_t) blk[1 + 2 * k] | ((uint32_t) blk[2 + 2 * k] << 16);
+                // block 2 q2 starts dword-aligned (its 16 nibble bytes straddle 5 dwords), block 2 q2 + 1 two bytes past a dword
+                // (its nibble bytes are 4 whole dwords)
+                {
+                    const int bb = 2 * q2;
+                    const uint32_t * pw = reinterpret_cast<const uint32_t *>(vs + key * C::HB + 18 * bb);
+                    const uint32_t d0 = pw[0], d1 = pw[1], d2 = pw[2], d3 = pw[3], d4 = pw[4];
+                    *reinterpret_cast<uint16_t *>(tab + bb * 32 + key * 2) = (uint16_t) d0;
+                    const u4 n = {__builtin_amdgcn_alignbit(d1, d0, 16), __builtin_amdgcn_alignbit(d2, d1, 16),
+                                  __builtin_amdgcn_alignbit(d3, d2, 16), __builtin_amdgcn_alignbit(d4, d3, 16)};
+                    *reinterpret_cast<u4 *>(va + key * 144 + 16 * bb) = n;
+                }
+                {
+                    const int bb = 2 * q2 + 1;
+                    const char * pb_ = vs + key * C::HB + 18 * bb;
+                    *reinterpret_cast<uint16_t *>(tab + bb * 32 + key * 2) = *reinterpret_cast<const uint16_t *>(pb_);
+                    const uint32_t * pw = reinterpret_cast<const uint32_t *>(pb_ + 2);
+                    const u4 n = {pw[0], pw[1], pw[2], pw[3]};
                     *reinterpret_cast<u4 *>(va + key * 144 + 16 * bb) = n;
                 }
             }
