@@ -136,12 +136,14 @@ template <int NR> __device__ __forceinline__ void wait_tiles(int newer) {
     else if (newer == 2) wait_vm_imm<2 * NR>();
     else wait_vm_imm<3 * NR>();
 }
+// A page-table entry through the scalar cache: a load from the constant address space at a wave-uniform address is an
+// s_load_dword, and the compiler itself places the wait for it before the first use of the value (a hand-written
+// s_load whose result the compiler may copy before a hand-written wait is a race). The table does not change while a
+// kernel runs.
 __device__ __forceinline__ int sload_i32(const int32_t * p) {
-    int v;
-    asm volatile("s_load_dword %0, %1, 0x0" : "=s"(v) : "s"(p));
-    return v;
+    return *reinterpret_cast<const __attribute__((address_space(4))) int32_t *>(rfl64((size_t) p));
 }
-__device__ __forceinline__ void wait_scalar(int & v) { asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(v)); }
+__device__ __forceinline__ void wait_scalar(int &) { }
 
 template <uint32_t KT, int D, int NT, int NWV, bool MULTI>
 __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const dec_params P) {
@@ -152,6 +154,11 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     __shared__ __attribute__((aligned(16))) char kv1[2 * NWV * C::SLOT_B];   // K slot 1, then V slot 1
     char * const kb1 = kv1, * const vb1 = kv1 + NWV * C::SLOT_B;
     static_assert(32 * D * 4 <= NWV * C::SLOT_B && 32 * C::QRS <= NWV * C::SLOT_B, "the Q copies (at most 32 columns) fit over the second K and V slots");
+    // q8_0 with two column tiles has no registers left for 64 dwords of Q operands (spills there cost more than their
+    // traffic: the compiler can only wait for a reload with "no vector memory operation outstanding", tiles included):
+    // that variant keeps the f16 Q table and reads its operands from it tile after tile
+    constexpr bool QLDS = KT == P1A_KV_Q8_0 && NT == 2;
+    __shared__ __attribute__((aligned(16))) char qtab[QLDS ? 32 * C::QRS : 16];
     __shared__ __attribute__((aligned(16))) char tabs[NWV * C::TAB_B];
     __shared__ __attribute__((aligned(16))) char vab[NWV * C::VA_B + 16];
 
@@ -217,6 +224,10 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             plim[r] = P.pos_rows ? P.pos_rows[row0 + t] : p0v + row0 + t;
         }
     }
+    // The limits are wanted HERE, before the first tile request: the compiler waits for its own loads with a plain
+    // "nothing outstanding", and placed after the requests such a wait would also wait for the tiles.
+#pragma unroll
+    for (int r = 0; r < NT; ++r) asm volatile("" : "+v"(plim[r]));
     const size_t head_off = (size_t) hk * C::HB;
     const int rowb = (int) P.pg.rowb;
 
@@ -288,16 +299,18 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     // what little work there is before the first tile is best kept short.)
     if (tile_start(0) < n_max) wait_vm_imm<2 * C::NRND>(); else wait_vm_imm<0>();
     __syncthreads();
-    for (int i = threadIdx.x; i < R * (D / 4); i += NWV * 64) {
+    char * const qt = QLDS ? qtab : vb1;
+    for (int i = threadIdx.x; i < (QLDS ? 32 : R) * (D / 4); i += NWV * 64) {
         const int col = i / (D / 4), d = 4 * (i - col * (D / 4));
-        const float4 a = *reinterpret_cast<const float4 *>(kb1 + (size_t) i * 16);
+        float4 a = make_float4(0.f, 0.f, 0.f, 0.f);          // (columns past the live ones: zero operands)
+        if (col < R) a = *reinterpret_cast<const float4 *>(kb1 + (size_t) i * 16);
         const float s = P.qscale;
-        *reinterpret_cast<h4 *>(vb1 + col * C::QRS + d * 2) = h4{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s)};
+        *reinterpret_cast<h4 *>(qt + col * C::QRS + d * 2) = h4{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s)};
     }
     __syncthreads();
-    h8 qf[NT][C::NMF];
+    h8 qf[QLDS ? 1 : NT][QLDS ? 1 : C::NMF];
 #pragma unroll
-    for (int r = 0; r < NT; ++r) {
+    for (int r = 0; r < (QLDS ? 0 : NT); ++r) {
         const int col = 16 * r + c;
         const bool livec = col < R;
         const char * qr = vb1 + (livec ? col : 0) * C::QRS;
@@ -394,8 +407,14 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
                 const u4 a0 = {x0.lo, x0.hi, x1.lo, x1.hi}, a1 = {x2.lo, x2.hi, x3.lo, x3.hi};
 #pragma unroll
                 for (int r = 0; r < NT; ++r) {
-                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a0), qf[r][2 * jj], s[r], 0, 0, 0);
-                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a1), qf[r][2 * jj + 1], s[r], 0, 0, 0);
+                    h8 q0, q1;
+                    if constexpr (QLDS) {   // operands 2 jj and 2 jj + 1 of column 16 r + c: 16 consecutive halves of its table row
+                        const char * qr = qtab + (16 * r + c) * C::QRS + 32 * (4 * jj + g);
+                        q0 = *reinterpret_cast<const h8 *>(qr);
+                        q1 = *reinterpret_cast<const h8 *>(qr + 16);
+                    } else { q0 = qf[r][2 * jj]; q1 = qf[r][2 * jj + 1]; }
+                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a0), q0, s[r], 0, 0, 0);
+                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a1), q1, s[r], 0, 0, 0);
                 }
                 if (have_n && jj < C::NRND) fetch_round(ksn, kn, tn, jj);
             }
@@ -561,41 +580,47 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         }
         __syncthreads();
         if (r == 0) TS(6);
-        const int items = Rr * (D / 4);
-        for (int it = threadIdx.x; it < items; it += NWV * 64) {
-            const int d4 = it % (D / 4), cc = it / (D / 4);
-            const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
-            const char * sbase = qtr == 0 ? kb0 : qtr == 1 ? kb1 : qtr == 2 ? vb0 : vb1;
-            // every LDS read first (they do not depend on one another), then the arithmetic; a wave that saw no visible
-            // key (m = -inf) parked zeros and gets the factor 0
-            float mw[NWV], lw[NWV];
-            f4 aw[NWV];
+        // 32 lanes per column: the factors of a column (one per wave; a wave that saw no visible key parked zeros and
+        // gets the factor 0) are worked out once per lane and serve all the dims the lane folds
+        constexpr int LPC = 32;
+        for (int cc = threadIdx.x / LPC; cc < Rr; cc += NWV * 64 / LPC) {
+            const int dl = threadIdx.x % LPC;
+            float mw[NWV], lw[NWV], fw[NWV];
 #pragma unroll
             for (int w = 0; w < NWV; ++w) {
                 const float * tw = reinterpret_cast<const float *>(tabs + w * C::TAB_B);
                 mw[w] = tw[cc];
                 lw[w] = tw[16 + cc];
-                aw[w] = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * C::QDP + dq);
             }
             float M = NEG_INF;
 #pragma unroll
             for (int w = 0; w < NWV; ++w) M = fmaxf(M, mw[w]);
-            f4 acc = {0.f, 0.f, 0.f, 0.f};
             float l = 0.f;
 #pragma unroll
             for (int w = 0; w < NWV; ++w) {
-                const float f = mw[w] == NEG_INF ? 0.f : __builtin_amdgcn_exp2f(mw[w] - M);
-                acc += aw[w] * f;
-                l += lw[w] * f;
+                fw[w] = mw[w] == NEG_INF ? 0.f : __builtin_amdgcn_exp2f(mw[w] - M);
+                l += lw[w] * fw[w];
             }
             const int col = 16 * r + cc;
             const int t = row_of(col), hh = col - t * P.GQA;
             const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) hg * P.GQA + hh;
-            // (two column tiles = several rows per group: the partials are tens of megabytes and nothing here reads them
-            // again, so they go past the cache - measured -3 ... -5 % on 4-row verify calls, +6 % on a single row)
-            f4 * const po = reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4);
-            if (M != NEG_INF) { if constexpr (NT == 2) __builtin_nontemporal_store(acc, po); else *po = acc; }
-            if (d4 == 0) {
+#pragma unroll
+            for (int d4 = dl; d4 < D / 4; d4 += LPC) {
+                const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
+                const char * sbase = qtr == 0 ? kb0 : qtr == 1 ? kb1 : qtr == 2 ? vb0 : vb1;
+                f4 aw[NWV];
+#pragma unroll
+                for (int w = 0; w < NWV; ++w)
+                    aw[w] = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * C::QDP + dq);
+                f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int w = 0; w < NWV; ++w) acc += aw[w] * fw[w];
+                // (two column tiles = several rows per group: the partials are tens of megabytes and nothing here reads
+                // them again, so they go past the cache - measured -3 ... -5 % on 4-row verify calls, +6 % on a single row)
+                f4 * const po = reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4);
+                if (M != NEG_INF) { if constexpr (NT == 2) __builtin_nontemporal_store(acc, po); else *po = acc; }
+            }
+            if (dl == 0) {
                 float * pm = P.part_ml + (row * P.nsplit + split) * 2;
                 pm[0] = M;
                 pm[1] = l;

@@ -158,6 +158,34 @@ def test_config3_batched_slots(p1a):
         assert torch.equal(one[0], out[t]), t
 
 
+def test_repeated_calls_give_the_same_bits(p1a):
+    """The same call repeated: bit-identical outputs every time (a page-table entry used before it had arrived once made
+    one call in a few differ), single row and 8 slots of unequal depth"""
+    Hq, Hkv, D, psh = 24, 4, 256, 8
+    lens = [8133, 19168, 27213, 2861, 6076, 9552, 23094, 1075]
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, psh, lens, seed=81, fill="device")
+    g = I.rng(82)
+    for s_, n in enumerate(lens):
+        c = pool.dev_seq(s_)
+        p1a.kv_append(c, dev(I.normal(g, (n, Hkv, D))), dev(I.normal(g, (n, Hkv, D))), 0, n)
+    dq = dev(I.normal(g, (8, Hq, D)))
+    pos = dev(np.array([n - 1 for n in lens], np.int32))
+    rt = dev(np.array([s_ * pool.maxp for s_ in range(8)], np.int32))
+    cr = pool.devkv.with_rows(rt)
+    ref8 = torch.empty((8, Hq, D), device="cuda")
+    p1a.attn_decode_rows(dq, cr, ref8, 8, pos, Hq, 1 / 16)
+    ref1 = torch.empty((1, Hq, D), device="cuda")
+    p1a.attn_decode(dq[2:3], pool.dev_seq(2), ref1, 1, lens[2] - 1, Hq, 1 / 16)
+    assert torch.equal(ref1[0], ref8[2])
+    for rep in range(150):
+        out8 = torch.full((8, Hq, D), float("nan"), device="cuda")
+        p1a.attn_decode_rows(dq, cr, out8, 8, pos, Hq, 1 / 16)
+        out1 = torch.full((1, Hq, D), float("nan"), device="cuda")
+        p1a.attn_decode(dq[2:3], pool.dev_seq(2), out1, 1, lens[2] - 1, Hq, 1 / 16)
+        assert torch.equal(out8, ref8), rep
+        assert torch.equal(out1, ref1), rep
+
+
 @pytest.mark.parametrize("kv_type", [O.KV_Q4_0, O.KV_Q8_0])
 def test_config4_verify_blocks(p1a, kv_type):
     """MTP verify: 4 sequences x 4 rows (1 accepted + 3 drafts), causal inside the block, f16-rounded inputs; context
