@@ -333,14 +333,18 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         gpages r;
         r.pg = 0;
         if (FAST && ptab) {
+            // (a load from the constant address space at a wave-uniform address is an s_load_dword whose wait the compiler
+            // places itself, before the first use; the table does not change while the kernel runs)
             const int32_t * e = ptab + (__builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, gclamp)) >> P.pg.psh);
-            asm volatile("s_load_dword %0, %1, 0x0" : "=s"(r.pg) : "s"(e));
+            const size_t eu = (size_t) e;
+            const uint32_t elo = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) eu);
+            const uint32_t ehi = (uint32_t) __builtin_amdgcn_readfirstlane((int) (uint32_t) (eu >> 32));
+            r.pg = *reinterpret_cast<const __attribute__((address_space(4))) int32_t *>(((size_t) ehi << 32) | elo);
         }
         return r;
     };
     auto group_bases = [&](int tile, gpages & gp) {
         gbases r;
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(gp.pg));
         const int p = __builtin_amdgcn_readfirstlane(min(tile * BN + 16 * wave, gclamp));
         r.go = (ptab ? (size_t) gp.pg * P.pg.pstride + (size_t) (p & pmask) * P.pg.rowb : (size_t) p * P.pg.rowb) + head_off;
         return r;
