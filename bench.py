@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the paged-KV attention hot path on one MI355X.
 
-Workload (N = 1): BASELINE.json configs[1] - 27B-shape decode, batch 1, one full-attention layer: 24 q heads / 4 kv
+Workload (N = 1): configs[1] of the baseline description - 27B-shape decode, batch 1, one full-attention layer: 24 q heads / 4 kv
 heads, head_dim 256, context 32768, q8_0 KV in 256-token pages scattered by a random permutation page table, fused
 sigmoid gate. A "step" is one p1a_attn_decode call (split-K kernel + merge) on inputs resident in HBM. The K timed
 steps are captured once into a hipGraph (the engine replays its decode step as a graph as well) and walk over several
@@ -88,7 +88,7 @@ def time_eager(torch, fn, reps, warmup=2):
 
 
 def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
-    """secondary measurements: the other BASELINE.json configs at full size (reported, not the headline value)"""
+    """secondary measurements: the other baseline configs at full size (reported, not the headline value)"""
     import math
     ex = {}
     g = torch.Generator(device="cuda").manual_seed(5)

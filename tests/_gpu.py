@@ -66,8 +66,12 @@ class Pool:
 
 
 def check(out, ref, what=""):
+    """max-abs <= 2e-3 (times max|ref| where the reference exceeds 1: the products run on f16 operands, whose error is
+    relative - the criterion of the engine's own tests, tests/fast_attn_test.cu:75,217,269 - and outputs above 1 only
+    occur for contexts of a few keys) and rel-L2 <= 1e-3"""
     ma, rl = I.errors(out, ref)
+    tol = I.MAX_ABS_TOL * max(1.0, float(np.max(np.abs(ref))))
     assert np.all(np.isfinite(out)), what
-    assert ma <= I.MAX_ABS_TOL and rl <= I.REL_L2_TOL, f"{what}: max_abs={ma:.3e} rel_l2={rl:.3e}"
-    print(f"[parity] {what}: max_abs={ma:.3e} (tol {I.MAX_ABS_TOL:g}) rel_l2={rl:.3e} (tol {I.REL_L2_TOL:g})")   # shown with pytest -s
+    assert ma <= tol and rl <= I.REL_L2_TOL, f"{what}: max_abs={ma:.3e} (tol {tol:.3g}) rel_l2={rl:.3e}"
+    print(f"[parity] {what}: max_abs={ma:.3e} (tol {tol:.3g}) rel_l2={rl:.3e} (tol {I.REL_L2_TOL:g})")   # shown with pytest -s
     return ma, rl

@@ -1,0 +1,89 @@
+"""Seeded sweeps over the shapes the C ABI accepts, each case against the CPU oracle (tolerance of the path: max-abs
+2e-3 - times max|ref| where a context of a few keys makes that exceed 1 - and rel-L2 1e-3): KV type, head counts, head dimension, page size, number of sequences, rows per sequence, lengths,
+gate on / off. The fixed-shape tests cover the engine's configurations; these look for a combination nobody thought of
+(ragged last pages, sequences shorter than a tile, a single key, page sizes below the MFMA kernels' minimum)."""
+import numpy as np
+import pytest
+import torch
+
+import _inputs as I
+import _oracle as O
+from _gpu import Pool, check, dev
+
+pytestmark = pytest.mark.gpu
+TYPES = [O.KV_F16, O.KV_Q8_0, O.KV_Q4_0]
+
+
+def draw_shape(g):
+    kv_type = TYPES[int(g.integers(3))]
+    D = int(g.choice([64, 128, 256], p=[0.2, 0.2, 0.6]))
+    Hkv = int(g.choice([1, 2, 3, 4]))
+    gqa = int(g.choice([1, 2, 4, 6, 8]))
+    psh = int(g.choice([2, 4, 5, 6, 8]))
+    return kv_type, D, Hkv, gqa, psh
+
+
+@pytest.mark.parametrize("case", range(40))
+def test_decode_random_case(p1a, case):
+    g = I.rng(9000 + case)
+    kv_type, D, Hkv, gqa, psh = draw_shape(g)
+    Hq = Hkv * gqa
+    nseq = int(g.integers(1, 5))
+    rps = int(g.integers(1, 5))
+    # lengths from one key up; every few cases a sequence that ends exactly on a page or tile boundary
+    lens = [max(rps, int(np.exp(g.uniform(0, np.log(2500))))) for _ in range(nseq)]
+    if case % 3 == 0:
+        lens[0] = max(rps, (lens[0] >> psh) << psh)
+    if case % 5 == 0:
+        lens[-1] = max(rps, (lens[-1] // 16) * 16 + 1)
+    use_gate = bool(g.integers(2))
+    scale = float(g.choice([1 / 16, 0.1, 0.125]))
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=9100 + case)
+    T = nseq * rps
+    q, _, _, gate = I.qkv(9200 + case, 1, T, Hq, Hkv, D)
+    pos = np.array([lens[s] - rps + t for s in range(nseq) for t in range(rps)], np.int32)
+    rtab = np.array([s * pool.maxp for s in range(nseq) for _ in range(rps)], np.int32)
+    ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, scale, gate=gate if use_gate else None)
+    out = torch.full((T, Hq, D), float("nan"), device="cuda")
+    what = f"decode case {case}: type {kv_type} {Hq}/{Hkv}/{D} psh {psh} lens {lens} rows/seq {rps} gate {use_gate}"
+    print(what, flush=True)
+    p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, T, dev(pos), Hq, scale,
+                         gate=dev(gate) if use_gate else None, rows_per_seq=rps)
+    torch.cuda.synchronize()
+    check(out.cpu().numpy(), ref, what)
+    # the first sequence alone, through the one-sequence entry (host position): the same bits as its rows in the batch
+    one = torch.full((rps, Hq, D), float("nan"), device="cuda")
+    p1a.attn_decode(dev(q[:rps]), pool.dev_seq(0), one, rps, lens[0] - rps, Hq, scale, gate=dev(gate[:rps]) if use_gate else None)
+    torch.cuda.synchronize()
+    assert torch.equal(one, out[:rps]), what
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_prefill_random_case(p1a, case):
+    g = I.rng(9500 + case)
+    kv_type, D, Hkv, gqa, psh = draw_shape(g)
+    Hq = Hkv * gqa
+    p0 = int(g.choice([0, int(g.integers(1, 1500))]))
+    T = int(np.exp(g.uniform(0, np.log(700)))) if case % 3 else int(g.integers(100, 600))
+    if case % 4 == 0:
+        T = max(1, (T // 128) * 128)                          # whole token blocks
+    use_gate = bool(g.integers(2))
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [p0 + T, 40], seed=9600 + case)
+    q, _, _, gate = I.qkv(9700 + case, 1, T, Hq, Hkv, D, f16_inputs=True)
+    pos = p0 + np.arange(T, dtype=np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, 0.1, gate=gate if use_gate else None)
+    what = f"prefill case {case}: type {kv_type} {Hq}/{Hkv}/{D} psh {psh} p0 {p0} T {T} gate {use_gate}"
+    print(what, flush=True)
+    c = pool.dev_seq(0)
+    out = torch.full((T, Hq, D), float("nan"), device="cuda")
+    p1a.attn_prefill(dev(q), c, out, T, p0, Hq, 0.1, gate=dev(gate) if use_gate else None)
+    torch.cuda.synchronize()
+    check(out.cpu().numpy(), ref, what)
+    # with caller scratch (a quantized cache converted once per call): the same bits
+    nb = p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D)
+    if nb:
+        scr = torch.empty(nb, dtype=torch.uint8, device="cuda")
+        out2 = torch.full((T, Hq, D), float("nan"), device="cuda")
+        p1a.attn_prefill(dev(q), c, out2, T, p0, Hq, 0.1, gate=dev(gate) if use_gate else None, scratch=scr)
+        torch.cuda.synchronize()
+        assert torch.equal(out, out2), what
