@@ -148,10 +148,11 @@ inline bool attn_prefill_variant(const float * q, const kv_cache & c, float * ou
                                  hipStream_t s, int /*variant: one kernel here*/) {
     return attn_prefill(q, c, out, T, p0, Hq, scale, s);
 }
-// src/fast/attn_fold.cuh:19-26 (chunk / nsplit are accepted and ignored: P never leaves the chip). The scratch is optional
+// src/fast/attn_fold.cuh:19-26 (chunk / nsplit are accepted and ignored: P never leaves the chip, and the library picks
+// the key splits of a short chunk over a long context itself, p1a_attn_prefill_key_splits). The scratch is optional
 // here: a buffer of attn_fold_scratch_bytes(T, Hkv, ..., p0) bytes lets a quantized cache be converted to f16 once per
-// call; the reference's own size (which knows nothing of p0) is accepted too and simply selects the on-the-fly kernel
-// when it is too small.
+// call and holds the split partials; the reference's own size (which knows nothing of p0) is accepted too: what does
+// not fit takes the on-the-fly kernel / the library's own buffers, with the same result bits.
 inline size_t attn_fold_scratch_bytes(int T, int Hkv, int /*chunk*/, int /*nsplit*/, int p0 = 0) {
     return p1a_attn_prefill_scratch_bytes(T, p0, 6 * Hkv, Hkv, 256);
 }

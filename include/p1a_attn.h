@@ -149,15 +149,23 @@ int p1a_ew_quant(int op, const float *a, const float *b, float *y, void *qbuf, i
  * fp16 MFMA products with fp32 accumulation; gate as in p1a_attn_decode. `scratch` is optional caller-supplied device
  * memory (256-byte aligned): with at least p1a_attn_prefill_scratch_bytes(...) bytes a q8_0 / q4_0 cache is converted to
  * f16 once per call instead of once per workgroup (same result bits, about 10-35 % less time); with less, or NULL, the
- * kernel converts on the fly. Rows of the cache past position p0 + T - 1 may be fetched (never past the end of a page,
+ * kernel converts on the fly. Results do not depend on the scratch passed. Rows of the cache past position p0 + T - 1 may be fetched (never past the end of a page,
  * or of a contiguous cache) but are never weighted, whatever they hold.
  * Replaces attn_prefill (src/fast/attn.cuh:46-50) and attn_fold (src/fast/attn_fold.cuh:19-26).
  */
 int p1a_attn_prefill(const float *q, const p1a_kv *c, float *out, const float *gate, int T, int p0, int Hq,
                      float scale, void *scratch, size_t scratch_bytes, void *stream);
-/* bytes of scratch that enable the convert-once variant: 2 * roundup(p0 + T, 16) * Hkv * D * 2. Replaces attn_fold_scratch_bytes
- * (src/fast/attn_fold.cuh:19). */
+/* bytes of scratch that enable the convert-once variant and hold the partials of a key-split call:
+ * roundup(2 * roundup(p0 + T, 16) * Hkv * D * 2, 256) + (key splits > 1 ? roundup(T * Hq * splits * 8, 256) + T * Hq * splits * D * 4 : 0).
+ * Replaces attn_fold_scratch_bytes (src/fast/attn_fold.cuh:19). */
 size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D);
+/* Key splits a prefill call of this shape takes on the current device (1 = none). A chunk of few token blocks over a long
+ * context (the last chunk of a prompt, a short turn of a long chat) would occupy T/128 * Hq workgroups, each walking every
+ * key; its keys are then dealt to several workgroups per (token block, q head) and the partials merged (the nsplit of
+ * attn_fold, src/fast/attn_fold.cuh:19-26, chosen by the library). The count depends on (T, p0, Hq) and the device's CU
+ * count only, never on the scratch passed; partials that do not fit the caller's scratch live in the library's own
+ * per-stream buffers (those of p1a_attn_decode; during stream capture they cannot grow and the call takes one split). */
+int p1a_attn_prefill_key_splits(int T, int p0, int Hq);
 
 /* Standalone sigmoid gate x[i] *= 1 / (1 + exp(-g[i])). Replaces k::sigmoid_mul, src/kernels.cu:85-93. */
 int p1a_sigmoid_mul(float *x, const float *g, size_t n, void *stream);

@@ -7,7 +7,7 @@ import os
 KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
-    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes",
+    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
     "p1a_version",
     # include/p1a_pool.h
@@ -79,6 +79,8 @@ def lib():
     L.p1a_attn_prefill.argtypes = [vp, kvp, vp, vp, i32, i32, i32, f32, vp, sz, vp]
     L.p1a_attn_prefill_scratch_bytes.restype = sz
     L.p1a_attn_prefill_scratch_bytes.argtypes = [i32, i32, i32, i32, i32]
+    L.p1a_attn_prefill_key_splits.restype = i32
+    L.p1a_attn_prefill_key_splits.argtypes = [i32, i32, i32]
     L.p1a_sigmoid_mul.restype = i32
     L.p1a_sigmoid_mul.argtypes = [vp, vp, sz, vp]
     L.p1a_warmup.restype = i32
@@ -281,6 +283,10 @@ def ew_quant(op, a, b, y, qbuf, T, n, lda=0, ldb=0):
 
 def prefill_scratch_bytes(T, p0, Hq, Hkv, D):
     return int(lib().p1a_attn_prefill_scratch_bytes(T, p0, Hq, Hkv, D))
+
+
+def prefill_key_splits(T, p0, Hq):
+    return int(lib().p1a_attn_prefill_key_splits(T, p0, Hq))
 
 
 def attn_prefill(q, c, out, T, p0, Hq, scale, gate=None, scratch=None):

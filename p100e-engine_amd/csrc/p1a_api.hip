@@ -33,6 +33,8 @@ int g_nsplit_override = 0;
 bool g_skip_merge = false;
 int g_cus[16] = {0};
 
+}   // namespace
+
 int cu_count() {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return 256;
@@ -41,28 +43,30 @@ int cu_count() {
     return n;
 }
 
-scratch * scratch_for(hipStream_t s, size_t need_o, size_t need_ml) {
+namespace {
+
+scratch * scratch_for(hipStream_t s, size_t need_o, size_t need_ml, bool quiet = false) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lk(g_mu);
     scratch * e = nullptr;
     for (int i = 0; i < g_nscr; ++i) if (g_scr[i].dev == dev && g_scr[i].s == s) e = &g_scr[i];
     if (!e) {
-        if (g_nscr == MAX_SCR) { set_error("too many (device, stream) pairs"); return nullptr; }
+        if (g_nscr == MAX_SCR) { if (!quiet) set_error("too many (device, stream) pairs"); return nullptr; }
         e = &g_scr[g_nscr++];
         e->dev = dev; e->s = s;
     }
     if (need_o > e->cap_o || need_ml > e->cap_ml) {
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         if (s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
-            set_error("split scratch would have to grow during stream capture: call p1a_warmup first");
+            if (!quiet) set_error("split scratch would have to grow during stream capture: call p1a_warmup first");
             return nullptr;
         }
         float * no = nullptr, * nm = nullptr;
         if (hipMalloc(&no, need_o) != hipSuccess || hipMalloc(&nm, need_ml) != hipSuccess) {
             (void) hipGetLastError();
             if (no) (void) hipFree(no);
-            set_error("split scratch allocation failed (%zu bytes)", need_o + need_ml);
+            if (!quiet) set_error("split scratch allocation failed (%zu bytes)", need_o + need_ml);
             return nullptr;
         }
         if (e->o) { (void) hipStreamSynchronize(s); (void) hipFree(e->o); (void) hipFree(e->ml); }
@@ -86,6 +90,14 @@ int nsplit_req() {
 }
 
 }   // namespace
+
+bool split_scratch(hipStream_t s, size_t bytes_o, size_t bytes_ml, float *& o, float *& ml) {
+    scratch * e = scratch_for(s, bytes_o, bytes_ml, true);
+    if (!e) return false;
+    o = e->o; ml = e->ml;
+    return true;
+}
+
 }   // namespace p1a
 
 using namespace p1a;

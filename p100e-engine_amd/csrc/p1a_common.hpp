@@ -109,6 +109,12 @@ int launch_prep(const p1a_kv & c, const float * qg, const float * k, const float
 int launch_ew_quant(int op, const float * a, const float * b, float * y, void * qbuf, int T, int n, int lda, int ldb, hipStream_t s);
 int launch_prefill(const p1a_kv & c, const float * q, float * out, const float * gate, int T, int p0, int Hq,
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s);
+// fold of split partials [rows][NS][D] + (m, l) [rows][NS][2] into out [rows][D] (rows = T * Hq), sigmoid gate fused
+int launch_merge(const float * part_o, const float * part_ml, float * out, const float * gate, int NS, int D, int Hq, int T, hipStream_t s);
+// the library's own split-partial buffers of (current device, stream), grown to at least these sizes; false (nothing
+// reported) when that is not possible now, e.g. the stream is being captured and the buffers would have to grow
+bool split_scratch(hipStream_t s, size_t bytes_o, size_t bytes_ml, float *& o, float *& ml);
+int cu_count();   // compute units of the current device
 int launch_sigmoid_mul(float * x, const float * g, size_t n, hipStream_t s);
 int launch_stream_read(const void * src, size_t bytes, hipStream_t s);   // benchmarks only
 

@@ -946,6 +946,11 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
+int launch_merge(const float * part_o, const float * part_ml, float * out, const float * gate, int NS, int D, int Hq, int T, hipStream_t s) {
+    merge_k<<<dim3((unsigned) T * Hq, D / 32), 64, 0, s>>>(part_o, part_ml, out, gate, NS, D, nullptr, Hq, T);
+    return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
+}
+
 #ifdef P1A_TRACE
 extern "C" void p1a_set_trace(long long * buf) { (void) hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &buf, sizeof buf); }
 #endif

@@ -82,6 +82,11 @@ struct pf_params {
     int n_rows;   // positions the cache holds (contiguous caches: rows that may be read)
     float qscale;
     int nblk;     // token blocks
+    // key splits: with nks > 1 workgroup (block, head, ks) walks its share of the block's tiles and leaves an unnormalised
+    // partial (O relative to m, and (m, l)) per row in part_o [T*Hq][nks][D] / part_ml [T*Hq][nks][2] for the merge
+    int nks;
+    float * part_o;
+    float * part_ml;
 };
 
 __device__ __forceinline__ uint32_t perm_b(uint32_t hi, uint32_t lo, uint32_t sel) { return __builtin_amdgcn_perm(hi, lo, sel); }
@@ -233,8 +238,11 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     const int c = lane & 31, g = lane >> 5;
     // blockIdx.x -> (token block, kv head, q head of the group): the GQA heads of one (block, kv head) share an XCD
     const int id = blockIdx.x, xcd = id & 7, slot = id >> 3;
-    const int unit = (slot / P.GQA) * 8 + xcd, hh = slot % P.GQA;
-    if (unit >= P.nblk * P.Hkv) return;
+    // (with key splits a unit is (key split, token block, kv head): the splits spread over the XCDs like the blocks do)
+    const int vunit = (slot / P.GQA) * 8 + xcd, hh = slot % P.GQA;
+    const int nunits = P.nblk * P.Hkv;
+    if (vunit >= nunits * P.nks) return;
+    const int ksp = vunit / nunits, unit = vunit - ksp * nunits;
     // longest blocks (most keys) first
     const int tb = P.nblk - 1 - unit / P.Hkv, hk = unit % P.Hkv;
     const int h = hk * P.GQA + hh;
@@ -248,7 +256,22 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     const int wave_pmin = P.p0 + wtok0;                       // smallest limit among this wave's rows
     const int wave_pmax = P.p0 + min(P.T - 1, wtok0 + 31);
     const bool wave_live = wtok0 < P.T;
-    const int ntiles = pmax / BN + 1;
+    const int ntiles_all = pmax / BN + 1;                     // tiles the block sees
+    // this workgroup's share of them: tiles tile_a .. tile_a + ntiles - 1
+    int tile_a = 0, ntiles = ntiles_all;
+    if (P.nks > 1) {
+        const int tps = (ntiles_all + P.nks - 1) / P.nks;
+        tile_a = ksp * tps;
+        ntiles = min(tps, ntiles_all - tile_a);
+        if (ntiles <= 0) {   // nothing left for this split: an empty partial (the merge skips it)
+            if (g == 0 && live) {
+                float * ml = P.part_ml + (((size_t) my_tok * P.Hq + h) * P.nks + ksp) * 2;
+                ml[0] = NEG_INF;
+                ml[1] = 0.f;
+            }
+            return;
+        }
+    }
 
     const int32_t * ptab = P.pg.pt ? (P.pg.rtab ? P.pg.pt + P.pg.rtab[0] : P.pg.pt) : nullptr;
     const size_t hb = KT == P1A_KV_F16 ? (size_t) D * 2 : KT == P1A_KV_Q8_0 ? (size_t) (D / 32) * 34 : (size_t) (D / 32) * 18;
@@ -304,7 +327,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     // rows past it (they would otherwise read rows nobody has written); that tile's offsets are prepared once, up front.
     constexpr bool grouped = GROUPED;
     const int pmask = (1 << P.pg.psh) - 1;
-    const int last_tile = ntiles - 1;
+    const int last_tile = ntiles_all - 1;                     // the tile that holds pmax
     using IM = item_map<S::CPK>;
     uint32_t voff[S::NPT][S::NOFF], voff_last[S::NPT][S::NOFF];
     int grp[S::NPT];                                             // (wave-major: all equal to the wave number)
@@ -427,7 +450,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     // the q heads of one group stay one tile apart, so all but the first still find the tile in L2.
     // Steps past the last one (the pipeline looks up to three tiles ahead) repeat the last tile; nothing uses them.
     const int rot = (int) (((unsigned) unit * 29u + (unsigned) hh) % (unsigned) ntiles);
-    auto tile_of = [&](int it) { const int t = min(it, last_tile) + rot; return t >= ntiles ? t - ntiles : t; };
+    auto tile_of = [&](int it) { const int t = min(it, ntiles - 1) + rot; return tile_a + (t >= ntiles ? t - ntiles : t); };
 
     // S^T of one tile: 32-key halves u = 0, 1
     auto qk = [&](const char * kt, f16x (&s)[2]) {
@@ -685,6 +708,26 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     // all 64 rows. Lane (row c, half g) holds dims 32 dt + 8 (i / 4) + 4 g + (i % 4) of tile dt ----
     if (g == 0) ax_own[c] = ol[0];
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");   // (also: no tile load is left in flight)
+    if (P.nks > 1) {   // one of several key splits: the unnormalised partial of every row, for the merge
+        if (g == 0 && live) {
+            float * ml = P.part_ml + (((size_t) my_tok * P.Hq + h) * P.nks + ksp) * 2;
+            ml[0] = m_run;
+            ml[1] = ol[0];
+        }
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int tok = tok0 + 32 * (r ? wave ^ 1 : wave) + c;
+            if (tok >= P.T) continue;
+            float * orow = P.part_o + (((size_t) tok * P.Hq + h) * P.nks + ksp) * D;
+#pragma unroll
+            for (int dt = 0; dt < HD; ++dt)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4)
+                    *reinterpret_cast<f4 *>(orow + 32 * (dh * HD + dt) + 8 * q4 + 4 * g) =
+                        f4{o[r][dt][4 * q4], o[r][dt][4 * q4 + 1], o[r][dt][4 * q4 + 2], o[r][dt][4 * q4 + 3]};
+        }
+        return;
+    }
     const float l_par = ax_par[c];
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
@@ -726,7 +769,7 @@ int launch_pf_g(const pf_params & P, hipStream_t s) {
         }
         attr_set.fetch_or(bit, std::memory_order_release);
     }
-    const int units = P.nblk * P.Hkv;
+    const int units = P.nblk * P.Hkv * P.nks;
     const int slots = ((units + 7) / 8) * P.GQA;
     prefill_k<KT, D, GROUPED, DMA><<<slots * 8, NTHR, lds, s>>>(P);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
@@ -795,6 +838,23 @@ __global__ void __launch_bounds__(256) dq_k(const char * kc, const char * vc, kv
 }
 }   // namespace
 
+// Key splits of a call: a chunk of few token blocks over a long context would leave most of the device idle (one
+// workgroup per block and q head, each walking every tile), so the tiles of a block are dealt to nks workgroups and the
+// partials merged. Chosen from the shape and the device alone (never from what scratch the caller brought: the result
+// bits depend on the split): the count that minimises rounds of workgroups x tiles per workgroup, a split being at least
+// 8 tiles and paying about 6 tiles' worth of set-up and partial traffic; 1 unless that saves 15 %.
+int prefill_key_splits(int T, int p0, int Hq, int cus) {
+    const long units = (long) ((T + BM - 1) / BM) * Hq, nt = (p0 + T - 1) / BN + 1;
+    if (cus < 1) cus = 1;
+    auto cost = [&](long k) { return ((units * k + cus - 1) / cus) * ((nt + k - 1) / k + 6); };
+    long best = 1, cbest = cost(1);
+    for (long k = 2; k <= 64 && nt / k >= 8; ++k)
+        if (cost(k) < cbest) { best = k; cbest = cost(k); }
+    return cbest * 100 <= cost(1) * 85 ? (int) best : 1;
+}
+size_t prefill_part_bytes_o(int T, int Hq, int D, int nks) { return nks > 1 ? (size_t) T * Hq * nks * D * 4 : 0; }
+size_t prefill_part_bytes_ml(int T, int Hq, int nks) { return nks > 1 ? (((size_t) T * Hq * nks * 2 * 4) + 255) & ~(size_t) 255 : 0; }
+
 // bytes of the f16 staging copy of the first n positions (K and V)
 // (rows rounded up to whole 16-key groups: the attention kernel fetches whole groups)
 size_t prefill_stage_bytes(int n, int Hkv, int D) { return 2 * (size_t) ((n + 15) & ~15) * Hkv * D * 2; }
@@ -809,14 +869,34 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
     P.n_rows = c.n_ctx;
     P.qscale = scale * 1.4426950408889634f;
     P.nblk = (T + BM - 1) / BM;
-#define PF(KT_) (c.D == 256 ? launch_pf<KT_, 256>(P, s) : c.D == 128 ? launch_pf<KT_, 128>(P, s) : launch_pf<KT_, 64>(P, s))
+    P.nks = 1; P.part_o = nullptr; P.part_ml = nullptr;
+    // the caller's scratch: first the f16 staging copy of a quantized cache (when it fits), then the split partials (when
+    // they fit behind it); partials that do not fit go to the library's own per-stream buffers
+    const int n = p0 + T;
+    static const bool no_stage = getenv("P1A_PF_NOSTAGE") && atoi(getenv("P1A_PF_NOSTAGE"));   // development A/B switch
+    static const int ks_env = getenv("P1A_PF_SPLIT") ? atoi(getenv("P1A_PF_SPLIT")) : 0;          // development A/B switch
+    const bool aligned = scratch && !((uintptr_t) scratch & 255);
+    const bool stage = c.type != P1A_KV_F16 && !no_stage && aligned && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D);
+    const size_t used = stage ? (prefill_stage_bytes(n, c.Hkv, c.D) + 255) & ~(size_t) 255 : 0;
+    int nks = ks_env > 0 ? ks_env : prefill_key_splits(T, p0, Hq, cu_count());
+    if (nks > 1) {
+        const size_t bo = prefill_part_bytes_o(T, Hq, c.D, nks), bm = prefill_part_bytes_ml(T, Hq, nks);
+        if (aligned && scratch_bytes >= used + bm + bo) {
+            P.part_ml = reinterpret_cast<float *>((char *) scratch + used);
+            P.part_o = reinterpret_cast<float *>((char *) scratch + used + bm);
+        } else if (!split_scratch(s, bo, bm, P.part_o, P.part_ml)) nks = 1;   // (no room anywhere, e.g. during stream capture)
+    }
+    P.nks = nks;
+    auto finish = [&](int rc) {
+        if (rc != P1A_OK || P.nks == 1) return rc;
+        return launch_merge(P.part_o, P.part_ml, out, gate, P.nks, c.D, Hq, T, s);
+    };
+#define PF(KT_) finish(c.D == 256 ? launch_pf<KT_, 256>(P, s) : c.D == 128 ? launch_pf<KT_, 128>(P, s) : launch_pf<KT_, 64>(P, s))
     if (c.type == P1A_KV_F16) return PF(P1A_KV_F16);
     // A quantized cache with enough caller scratch: convert the visible positions to f16 once (tens of microseconds, the
     // copy stays in the Infinity Cache) and run the f16 kernel on it - every workgroup then skips the dequantization it
     // would otherwise repeat per 128 query rows. Same tiles, same products, same bits as the direct kernel.
-    const int n = p0 + T;
-    static const bool no_stage = getenv("P1A_PF_NOSTAGE") && atoi(getenv("P1A_PF_NOSTAGE"));   // development A/B switch
-    if (!no_stage && scratch && !((uintptr_t) scratch & 255) && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D)) {
+    if (stage) {
         const int n16 = (n + 15) & ~15;
         char * ko = (char *) scratch, * vo = ko + (size_t) n16 * c.Hkv * c.D * 2;
         const long long items = (long long) n * (c.Hkv * c.D / (c.type == P1A_KV_Q8_0 ? 16 : 32));
@@ -842,9 +922,16 @@ extern "C" void p1a_set_pf_trace(long long * buf) { (void) hipMemcpyToSymbol(HIP
 #endif
 
 extern "C" size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D) {
-    (void) Hq;
     if (T < 1 || p0 < 0 || Hkv < 1 || D < 1) return 0;
     // optional: with this much scratch a quantized cache is converted to f16 once per call instead of once per
-    // workgroup; with less (or none) the kernel converts on the fly and needs nothing
-    return p1a::prefill_stage_bytes(p0 + T, Hkv, D);
+    // workgroup, and the partials of a key-split call (few token blocks over a long context) live in it; with less (or
+    // none) the kernel converts on the fly and the partials go to the library's own per-stream buffers
+    const int nks = Hq >= 1 ? p1a::prefill_key_splits(T, p0, Hq, p1a::cu_count()) : 1;
+    return ((p1a::prefill_stage_bytes(p0 + T, Hkv, D) + 255) & ~(size_t) 255) + p1a::prefill_part_bytes_ml(T, Hq, nks) +
+           p1a::prefill_part_bytes_o(T, Hq, D, nks);
+}
+
+extern "C" int p1a_attn_prefill_key_splits(int T, int p0, int Hq) {
+    if (T < 1 || p0 < 0 || Hq < 1) return 1;
+    return p1a::prefill_key_splits(T, p0, Hq, p1a::cu_count());
 }

@@ -93,9 +93,12 @@ def test_scratch_variant_gives_the_same_bits(p1a, kv_type, Hq, Hkv, D, psh):
     q, _, _, gate = I.qkv(70 + D, 1, T, Hq, Hkv, D, f16_inputs=True)
     a = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16, gate=gate)
     need = p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D)
-    assert need == 2 * ((p0 + T + 15) // 16 * 16) * Hkv * D * 2       # whole 16-key groups of f16 rows, K and V
+    stage = 2 * ((p0 + T + 15) // 16 * 16) * Hkv * D * 2               # whole 16-key groups of f16 rows, K and V
+    ks = p1a.prefill_key_splits(T, p0, Hq)                            # (this shape is split over the keys)
+    r256 = lambda x: (x + 255) // 256 * 256
+    assert need == r256(stage) + (r256(T * Hq * ks * 8) + T * Hq * ks * D * 4 if ks > 1 else 0)
     dq, dg = dev(q), dev(gate)
-    for nbytes in (need, need // 2):
+    for nbytes in (need, r256(stage), stage // 2):                    # everything fits / the copy only / nothing
         scr = torch.full((nbytes,), 0xff, dtype=torch.uint8, device="cuda")   # (what the copy does not write is NaN)
         out = torch.zeros((T, Hq, D), device="cuda")
         p1a.attn_prefill(dq, pool.dev_seq(0), out, T, p0, Hq, 1 / 16, gate=dg, scratch=scr)
@@ -156,3 +159,49 @@ def test_f16_contiguous_and_small_pages_take_the_same_bits(p1a):
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
     ma, rl = I.errors(outs[0], want)
     assert ma < 2e-3 and rl < 1e-3, (ma, rl)
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("Hq,Hkv,D,p0,T", [(4, 1, 256, 6000, 100), (6, 2, 256, 9000, 260), (8, 2, 128, 5000, 70), (24, 4, 256, 12000, 33)])
+def test_key_split_chunks(p1a, kv_type, Hq, Hkv, D, p0, T):
+    """a short chunk over a long context is split over the keys (several workgroups per token block and head, partials
+    merged): against the oracle; every 7th row against the decode kernel at its position; and the same bits wherever the
+    partials live (caller scratch, the library's buffers) and whatever else is in flight before"""
+    ks = p1a.prefill_key_splits(T, p0, Hq)
+    assert ks > 1, ks
+    psh = 6
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [p0 + T], seed=p0 + T)
+    q, _, _, gate = I.qkv(p0, 1, T, Hq, Hkv, D, f16_inputs=True)
+    pos = p0 + np.arange(T, dtype=np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, 1 / 16, gate=gate)
+    c = pool.dev_seq(0)
+    out = run_prefill(p1a, c, q, T, p0, Hq, 1 / 16, gate=gate)
+    check(out, ref, f"key-split prefill type {kv_type} {Hq}/{Hkv}/{D} p0 {p0} T {T} splits {ks}")
+    dq, dg = dev(q), dev(gate)
+    need = p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D)
+    for nbytes in (need, need - 256, 4096):
+        scr = torch.full((nbytes,), 0xff, dtype=torch.uint8, device="cuda")
+        o2 = torch.zeros((T, Hq, D), device="cuda")
+        p1a.attn_prefill(dq, c, o2, T, p0, Hq, 1 / 16, gate=dg, scratch=scr)
+        torch.cuda.synchronize()
+        assert np.array_equal(o2.cpu().numpy(), out), nbytes
+    for t in range(0, T, 7):
+        one = torch.zeros((1, Hq, D), device="cuda")
+        p1a.attn_decode(dq[t:t + 1], c, one, 1, p0 + t, Hq, 1 / 16, gate=dg[t:t + 1])
+        ma, rl = I.errors(one.cpu().numpy()[0], out[t])
+        assert ma < 2e-3 and rl < 1e-3, (t, ma, rl)
+
+
+def test_key_split_plan():
+    """the split count is a function of the shape and the device only: none for chunks that fill the device or contexts too
+    short to share out, several for a short chunk over a long context; the scratch size says what it holds"""
+    import importlib
+    p1a = importlib.import_module("p100e-engine_amd")
+    assert p1a.prefill_key_splits(4096, 28672, 24) == 1             # the benchmark chunk: 768 workgroups already
+    assert p1a.prefill_key_splits(128, 0, 24) == 1                  # two tiles: nothing to share out
+    assert p1a.prefill_key_splits(64, 511, 4) == 1                  # splits of fewer than 8 tiles are not worth their set-up
+    assert p1a.prefill_key_splits(128, 32640, 24) >= 8
+    assert p1a.prefill_key_splits(512, 32256, 24) >= 2
+    for T, p0, Hq in [(128, 32640, 24), (33, 12000, 24), (300, 777, 12)]:
+        ks = p1a.prefill_key_splits(T, p0, Hq)
+        assert (p0 + T - 1) // 64 + 1 >= 8 * ks or ks == 1

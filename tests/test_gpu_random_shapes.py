@@ -87,3 +87,45 @@ def test_prefill_random_case(p1a, case):
         p1a.attn_prefill(dev(q), c, out2, T, p0, Hq, 0.1, gate=dev(gate) if use_gate else None, scratch=scr)
         torch.cuda.synchronize()
         assert torch.equal(out, out2), what
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_append_random_case(p1a, case):
+    """quantize-on-append into a paged pool in chunks of random size through the three position forms (host p0, device
+    p0, one position per row): every byte of the pool as the oracle writes it. Magnitudes from 1e-7 (scales that are f16
+    subnormals or underflow to zero) to 3e4 (close to the largest f16 scale), zero blocks and rows sprinkled in."""
+    g = I.rng(9800 + case)
+    kv_type = TYPES[int(g.integers(3))]
+    Hkv = int(g.choice([1, 2, 3, 4]))
+    D = int(g.choice([32, 64, 96, 128, 256]))
+    psh = int(g.choice([0, 2, 4, 5, 8]))
+    lens = [int(np.exp(g.uniform(0, np.log(900)))) if i else int(g.integers(100, 700)) for i in range(int(g.integers(1, 4)))]
+    pool = Pool(p1a, kv_type, Hkv, Hkv, D, psh, lens, seed=9900 + case, n_layers=int(g.integers(1, 4)), layer=0, fill="none")
+    what = f"append case {case}: type {kv_type} Hkv {Hkv} D {D} psh {psh} lens {lens}"
+    print(what, flush=True)
+    p0d = dev(np.array([0], np.int32))
+    for s, n in enumerate(lens):
+        mag = np.exp(g.uniform(np.log(1e-7), np.log(3e4), size=(n, Hkv, D // 32, 1))).astype(np.float32)
+        k = (I.normal(g, (n, Hkv, D // 32, 32)) * mag).reshape(n, Hkv, D)
+        v = (I.normal(g, (n, Hkv, D // 32, 32)) * mag[::-1]).reshape(n, Hkv, D)
+        k[g.integers(n)] = 0.0
+        v[g.integers(n), g.integers(Hkv), :32] = 0.0
+        O.kv_append_rows(pool.host.view(rtab=np.full(n, s * pool.maxp, np.int32)), k, v, np.arange(n))
+        dk, dv, c = dev(k), dev(v), pool.dev_seq(s)
+        a = 0
+        while a < n:
+            m = min(n - a, int(g.integers(1, 200)))
+            form = int(g.integers(3))
+            if form == 0:
+                p1a.kv_append(c, dk[a:], dv[a:], a, m)
+            elif form == 1:
+                p0d.fill_(a)
+                p1a.kv_append_dev(c, dk[a:], dv[a:], p0d, m)
+            else:   # rows in a shuffled order, through the row table
+                order = g.permutation(m)
+                cr = pool.devkv.with_rows(dev(np.full(m, s * pool.maxp, np.int32)))
+                idx = torch.from_numpy(a + order).cuda()
+                p1a.kv_append_rows(cr, dk[idx].contiguous(), dv[idx].contiguous(), dev((a + order).astype(np.int32)), m)
+            a += m
+    torch.cuda.synchronize()
+    assert np.array_equal(pool.dpool.cpu().numpy(), pool.host.pool), what
