@@ -117,6 +117,14 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
     sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=5)
     ex["prefill_no_scratch_ms"] = round(sec * 1e3, 4)
     del scr
+    # a short last chunk over the same context: its keys are split over several workgroups per (token block, head)
+    Ts, p0s = 128, p0 + T - 128
+    scr = torch.empty(p1a.prefill_scratch_bytes(Ts, p0s, Hq, Hkv, D), dtype=torch.uint8, device="cuda")
+    sec = time_eager(torch, lambda: p1a.attn_prefill(q[:Ts], c, out[:Ts], Ts, p0s, Hq, scale, gate=gate[:Ts], scratch=scr), reps=10)
+    ex["prefill_T128_p32640_q8_0_us"] = round(sec * 1e6, 1)
+    ex["prefill_T128_key_splits"] = p1a.prefill_key_splits(Ts, p0s, Hq)
+    ex["prefill_T128_TFLOPs"] = round(4.0 * D * Hq * (p0s * Ts + Ts * (Ts + 1) / 2) / sec / 1e12, 1)
+    del scr
     sec = time_eager(torch, lambda: p1a.kv_append(c, kc, vc, p0, T), reps=20)
     ab = 2 * T * Hkv * D * 4 + 2 * T * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
     ex["append_T4096_q8_0_us"] = round(sec * 1e6, 2)
