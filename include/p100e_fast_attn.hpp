@@ -63,6 +63,13 @@ inline kv_cache kv_alloc(uint32_t type, int n_ctx, int Hkv, int D) {
     return c;
 }
 
+// src/fast/attn.cuh:70 (attn.cu:559-581): benchmark fill of positions p0 .. p1 - 1, the same bytes for the same seed
+inline void kv_fill_random(kv_cache & c, int p0, int p1, uint32_t seed, hipStream_t s) {
+    if (!c.k || p1 <= p0) return;
+    const p1a_kv p = detail::pod(c);
+    (void) p1a_kv_fill_random(&p, p0, p1, seed, s);
+}
+
 // src/fast/attn.cuh:37-38
 inline void kv_append(kv_cache & c, const float * k, const float * v, int p0, int T, hipStream_t s) {
     const p1a_kv p = detail::pod(c);

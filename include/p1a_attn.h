@@ -80,6 +80,15 @@ int p1a_kv_append(const p1a_kv *c, const float *k, const float *v, int p0, const
                   const int32_t *pos_rows, int T, void *stream);
 
 /*
+ * Benchmark fill: positions p0 .. p1 - 1 of ONE sequence (page table pt + (rtab ? rtab[0] : 0), or contiguous) get hashed
+ * 16-bit words - f16 values in [-1, 1], or random codes under constant block scales (q8_0 1/127, q4_0 0.125) - the same
+ * bytes the reference writes for the same seed. The page table is read on the device (the reference copies it back).
+ * Replaces kv_fill_random (src/fast/attn.cuh:70, attn.cu:538-581), which the engine's bench_fill_kv calls
+ * (src/tp_model.cu:3195-3209).
+ */
+int p1a_kv_fill_random(const p1a_kv *c, int p0, int p1, uint32_t seed, void *stream);
+
+/*
  * Attention-layer input prep in one launch: per token t
  *     qg [T][ldq] (Hq heads, each D floats of q followed by D floats of gate) -> gate [T][Hq*D] (copy) and
  *                                                                                q [T][Hq][D] = rope(rmsnorm(q) * q_norm)

@@ -285,6 +285,56 @@ int orc_attn_prep_mrope(const float *qg, const float *k, const float *v, const f
 }
 
 /*
+ * Benchmark fill (src/fast/attn.cu:538-557 fill_random_k, :559-581 kv_fill_random). The cache is taken as 16-bit words;
+ * word w (index inside the contiguous cache, or inside the page for a paged one) gets
+ *   h = (uint32) w * 2654435761 ^ seed;  h ^= h >> 16;  h *= 0x7feb352d;  h ^= h >> 15;  h *= 0x846ca68b;  h ^= h >> 16
+ *   f16:  K = f16((h & 0xffff) / 32768 - 1), V = f16((h >> 16) / 32768 - 1)
+ *   scale words (q8_0: the first D/32 words of a head row; q4_0: every 9th word): f16(1/127) resp. f16(0.125), K and V
+ *   other words: K = low half of h, V = high half.
+ * Paged: logical page g of the sequence is filled as a contiguous cache at its page base with seed + g * 0x632be5ab.
+ */
+static void fill_words(uint16_t *k, uint16_t *v, size_t w0, size_t nw, uint32_t type, int D, int head_words, uint32_t seed) {
+    for (size_t i = 0; i < nw; ++i) {
+        const size_t w = w0 + i;
+        uint32_t h = (uint32_t) w * 2654435761u ^ seed;
+        h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+        const int hw = (int) (w % (size_t) head_words);
+        uint16_t a, b;
+        if (type == ORC_KV_F16) {
+            a = orc_f32_to_f16((float) (h & 0xffffu) / 32768.0f - 1.0f);
+            b = orc_f32_to_f16((float) (h >> 16) / 32768.0f - 1.0f);
+        } else if ((type == ORC_KV_Q8_0 && hw < D / 32) || (type == ORC_KV_Q4_0 && hw % 9 == 0)) {
+            a = b = orc_f32_to_f16(type == ORC_KV_Q8_0 ? 1.0f / 127.0f : 0.125f);
+        } else {
+            a = (uint16_t) h;
+            b = (uint16_t) (h >> 16);
+        }
+        k[w] = a;
+        v[w] = b;
+    }
+}
+
+void orc_kv_fill_random(const orc_kv *c, int p0, int p1, uint32_t seed) {
+    if (!c->k || p1 <= p0) return;
+    const size_t rowb = orc_kv_row_bytes(c->type, c->Hkv, c->D);
+    const int head_words = (int) (rowb / c->Hkv / 2);
+    if (!c->pt) {
+        fill_words((uint16_t *) c->k, (uint16_t *) c->v, (size_t) p0 * rowb / 2, (size_t) (p1 - p0) * rowb / 2, c->type, c->D, head_words, seed);
+        return;
+    }
+    const int32_t *pt = c->pt + (c->rtab ? c->rtab[0] : 0);
+    const int ps = 1 << c->psh;
+    for (int a = p0; a < p1;) {
+        const int pg = a >> c->psh, b = p1 < (pg + 1) * ps ? p1 : (pg + 1) * ps;
+        uint16_t *kp = (uint16_t *) ((uint8_t *) c->k + (size_t) pt[pg] * c->pstride);
+        uint16_t *vp = (uint16_t *) ((uint8_t *) c->v + (size_t) pt[pg] * c->pstride);
+        fill_words(kp, vp, (size_t) (a - pg * ps) * rowb / 2, (size_t) (b - a) * rowb / 2, c->type, c->D, head_words,
+                   seed + (uint32_t) pg * 0x632be5abu);
+        a = b;
+    }
+}
+
+/*
  * a16 activation quantize of the engine's quantized matvec (src/fast/matvec_a16.cu:29-100 quantize_a16, restated for
  * fused producers in src/fast/a16q.cuh:21-45): per token row t of n values, per group g of 32 values
  *   amax = max |v| (clamped to 65504 when it would round to an infinite f16), id = amax > 0 ? 1 / amax : 0,

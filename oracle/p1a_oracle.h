@@ -22,6 +22,10 @@
  *       and [2, 1, 1, 0]; moving one stream changes exactly the pairs of that stream.
  *   orc_a16_quant                              : an independent numpy float32 restatement (element -> slot map written out
  *       from the engine's comment, not from its index arithmetic), closed forms (zero group, unit group, clamp at 65520).
+ *   orc_kv_fill_random                         : the reference holds no vectors for its benchmark fill; pinned by the two
+ *       fixed points of its word hash (word 0 / seed 0 and word 1 / seed = the multiplier both hash to 0, hence f16 -1.0
+ *       or code 0), a big-integer restatement of the hash written out step by step, the places and bits of the scale
+ *       words, the value range, additivity over position ranges and paged == page-by-page contiguous with the page seeds.
  * No function of this file is "parity unpinned".
  */
 #ifndef P1A_ORACLE_H
@@ -90,6 +94,9 @@ int orc_attn_prep_mrope(const float *qg, const float *k, const float *v, const f
 /* a16 activation quantize (src/fast/a16q.cuh:21-45 = src/fast/matvec_a16.cu:29-100): y [T][n] f32, n % 32 == 0 ->
  * qbuf: T * n/32 * 16 half2 of scaled values (slot order of the engine), then T * n/32 half2 (amax, sum). */
 void orc_a16_quant(const float *y, int T, int n, uint16_t *qbuf);
+/* benchmark fill of positions p0 .. p1 - 1 of ONE sequence (page table pt + (rtab ? rtab[0] : 0)) with hashed 16-bit
+ * words: src/fast/attn.cu:538-581 (kv_fill_random; the engine's bench_fill_kv, src/tp_model.cu:3195-3209, calls it). */
+void orc_kv_fill_random(const orc_kv *c, int p0, int p1, uint32_t seed);
 int orc_num_threads(void);
 
 #ifdef __cplusplus

@@ -7,7 +7,7 @@ import os
 KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
-    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
+    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_kv_fill_random", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
     "p1a_version",
     # include/p1a_pool.h
@@ -79,6 +79,8 @@ def lib():
     L.p1a_attn_prefill.argtypes = [vp, kvp, vp, vp, i32, i32, i32, f32, vp, sz, vp]
     L.p1a_attn_prefill_scratch_bytes.restype = sz
     L.p1a_attn_prefill_scratch_bytes.argtypes = [i32, i32, i32, i32, i32]
+    L.p1a_kv_fill_random.restype = i32
+    L.p1a_kv_fill_random.argtypes = [kvp, i32, i32, ctypes.c_uint32, vp]
     L.p1a_attn_prefill_key_splits.restype = i32
     L.p1a_attn_prefill_key_splits.argtypes = [i32, i32, i32]
     L.p1a_sigmoid_mul.restype = i32
@@ -229,6 +231,11 @@ class KVCache:
 def kv_append(c, k, v, p0, T):
     """src/fast/attn.cuh:37-38 of the reference: k, v [T][Hkv][D] f32 -> cache positions p0..p0+T-1."""
     _check(lib().p1a_kv_append(ctypes.byref(c.struct()), _ptr(k), _ptr(v), p0, None, None, T, _stream()), "kv_append")
+
+
+def kv_fill_random(c, p0, p1, seed):
+    """src/fast/attn.cuh:70: benchmark fill of positions p0 .. p1 - 1 of one sequence."""
+    _check(lib().p1a_kv_fill_random(ctypes.byref(c.struct()), p0, p1, seed & 0xffffffff, _stream()), "kv_fill_random")
 
 
 def kv_append_dev(c, k, v, p0_dev, T):

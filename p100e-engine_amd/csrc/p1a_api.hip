@@ -119,6 +119,15 @@ int p1a_kv_append(const p1a_kv * c, const float * k, const float * v, int p0, co
     return launch_append(*c, k, v, p0, p0_dev, pos_rows, T, (hipStream_t) stream);
 }
 
+int p1a_kv_fill_random(const p1a_kv * c, int p0, int p1, uint32_t seed, void * stream) {
+    if (!kv_ok(c, "p1a_kv_fill_random")) return P1A_E_ARG;
+    if (p0 < 0) { set_error("p1a_kv_fill_random: negative p0"); return P1A_E_ARG; }
+    if (p1 <= p0) return P1A_OK;
+    if (c->type != P1A_KV_F16 && c->D % 32) { set_error("p1a_kv_fill_random: D %% 32 != 0"); return P1A_E_SHAPE; }
+    if (!c->pt && p1 > c->n_ctx) { set_error("p1a_kv_fill_random: positions up to %d in a cache of %d", p1, c->n_ctx); return P1A_E_ARG; }
+    return launch_fill_random(*c, p0, p1, seed, (hipStream_t) stream);
+}
+
 int p1a_attn_prep(const float * qg, const float * k, const float * v, const float * q_norm, const float * k_norm,
                   const int32_t * pos, float * q, float * gate, const p1a_kv * c, int p0, int T, int Hq, int n_rot,
                   float freq_base, float eps, int ldq, int ldk, int ldv, void * stream) {

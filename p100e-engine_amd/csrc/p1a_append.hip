@@ -230,6 +230,53 @@ int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, co
 }
 
 namespace {
+// Benchmark fill of positions p0 .. p1 - 1 of one sequence with hashed 16-bit words (src/fast/attn.cu:538-581): word w of
+// the contiguous cache - or of the page, for a paged one, whose logical page g then adds g * 0x632be5ab to the seed - gets
+// a 32-bit mix of (w, seed); f16 caches take its halves as values in [-1, 1], the quantized ones as codes, with every
+// scale word set to f16(1/127) (q8_0) or f16(0.125) (q4_0). The page table is read on the device: nothing is copied back
+// to the host, and the call can be captured.
+__global__ void __launch_bounds__(256) fill_random_k(uint16_t * kc, uint16_t * vc, kv_view pg, uint32_t type, int D, int p0, size_t nw,
+                                                     int row_words, int head_words, uint32_t seed) {
+    const int32_t * ptab = pg.pt ? (pg.rtab ? pg.pt + pg.rtab[0] : pg.pt) : nullptr;
+    for (size_t i = (size_t) blockIdx.x * 256 + threadIdx.x; i < nw; i += (size_t) gridDim.x * 256) {
+        const int p = p0 + (int) (i / (size_t) row_words), wr = (int) (i % (size_t) row_words);
+        size_t w, base = 0;                                   // word index the hash takes; where that view starts (bytes)
+        uint32_t sd = seed;
+        if (ptab) {
+            const int g = p >> pg.psh;
+            w = (size_t) (p - (g << pg.psh)) * row_words + wr;
+            base = (size_t) ptab[g] * pg.pstride;
+            sd = seed + (uint32_t) g * 0x632be5abu;
+        } else w = (size_t) p * row_words + wr;
+        uint32_t h = (uint32_t) w * 2654435761u ^ sd;
+        h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+        const int hw = wr % head_words;
+        uint16_t a, b;
+        if (type == P1A_KV_F16) {
+            a = __builtin_bit_cast(uint16_t, (half_t) ((float) (h & 0xffffu) / 32768.0f - 1.0f));
+            b = __builtin_bit_cast(uint16_t, (half_t) ((float) (h >> 16) / 32768.0f - 1.0f));
+        } else if ((type == P1A_KV_Q8_0 && hw < D / 32) || (type == P1A_KV_Q4_0 && hw % 9 == 0)) {
+            a = b = __builtin_bit_cast(uint16_t, (half_t) (type == P1A_KV_Q8_0 ? 1.0f / 127.0f : 0.125f));
+        } else {
+            a = (uint16_t) h;
+            b = (uint16_t) (h >> 16);
+        }
+        reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(kc) + base)[w] = a;
+        reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(vc) + base)[w] = b;
+    }
+}
+}   // namespace
+
+int launch_fill_random(const p1a_kv & c, int p0, int p1, uint32_t seed, hipStream_t s) {
+    const size_t rowb = p1a_kv_row_bytes(c.type, c.Hkv, c.D);
+    const int row_words = (int) (rowb / 2), head_words = row_words / c.Hkv;
+    const size_t nw = (size_t) (p1 - p0) * row_words;
+    const unsigned blocks = (unsigned) (nw / 256 + 1 < 4096 ? nw / 256 + 1 : 4096);
+    fill_random_k<<<blocks, 256, 0, s>>>((uint16_t *) c.k, (uint16_t *) c.v, view_of(c), c.type, c.D, p0, nw, row_words, head_words, seed);
+    return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
+}
+
+namespace {
 // elementwise gate + a16 quantize, one float4 per lane, 8 lanes per 32-value group (src/fast/fused.cu:478-496):
 // OP 0: y = silu(a) * b (the MLP gate); OP 1: y = a * sigmoid(b) (the attention output gate). y may alias a.
 template <int OP>

@@ -50,6 +50,21 @@ constexpr size_t head_bytes(uint32_t type, int D) {
 // T * ng * 16 + t * ng + g = (amax, sum of the scaled values). Products and sums are rounded one by one (no contraction),
 // the sum runs over a lane's 4 values in order from +0 and then over the lanes in an xor butterfly with strides 4, 2, 1.
 #if defined(__HIPCC__)
+// v_permlane16_swap / v_permlane32_swap exchange the odd 16-lane rows (the upper 32 lanes) of the first register with the
+// even rows (the lower 32 lanes) of the second; BOTH registers are results. They are issued through inline assembly: the
+// compiler's builtin for them hands back its first result twice (the second register - the other half of the exchange -
+// is dropped), so a maximum built on it silently kept the even rows' / lower lanes' value only. The instruction needs two
+// wait states after a vector write of either operand, which the compiler does not know to insert around assembly; the maximum of the two results rides in the same block.
+__device__ __forceinline__ float max_swap16(float m) {
+    float a = m, b = m;
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 0\n\tv_max_f32 %0, %0, %1" : "+v"(a), "+v"(b));
+    return a;
+}
+__device__ __forceinline__ float max_swap32(float m) {
+    float a = m, b = m;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 0\n\tv_max_f32 %0, %0, %1" : "+v"(a), "+v"(b));
+    return a;
+}
 __device__ __forceinline__ void a16_quant8(const f4 v4, int l8, void * qbuf, int t, int g, int ng, int T, bool store) {
 #pragma clang fp contract(off)
     float v[4] = {v4[0], v4[1], v4[2], v4[3]};
@@ -78,6 +93,8 @@ __device__ __forceinline__ void a16_quant8(const f4 v4, int l8, void * qbuf, int
 // host-side launch entry points implemented in the .hip files
 int launch_append(const p1a_kv & c, const float * k, const float * v, int p0, const int32_t * p0_dev,
                   const int32_t * pos_rows, int T, hipStream_t s);
+
+int launch_fill_random(const p1a_kv & c, int p0, int p1, uint32_t seed, hipStream_t s);
 
 struct decode_args {
     const float * q;

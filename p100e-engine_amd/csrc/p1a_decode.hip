@@ -97,12 +97,7 @@ __device__ __forceinline__ u2 deq4(uint32_t w, h2 d01, h2 d23) {
 }
 
 // the maximum over the four lanes that share (lane & 15): the two 16-lane rows of each half, then the two halves
-__device__ __forceinline__ float max_over_groups(float m) {
-    const auto a = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, m), __builtin_bit_cast(unsigned, m), false, false);
-    m = fmaxf(__builtin_bit_cast(float, a[0]), __builtin_bit_cast(float, a[1]));
-    const auto b = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, m), __builtin_bit_cast(unsigned, m), false, false);
-    return fmaxf(__builtin_bit_cast(float, b[0]), __builtin_bit_cast(float, b[1]));
-}
+__device__ __forceinline__ float max_over_groups(float m) { return max_swap32(max_swap16(m)); }
 
 // 4 nibbles (the low nibbles of the 4 bytes of w) -> ((n - 8) * d) as two packed f16 pairs (0x6400 | n = 1024 + n)
 __device__ __forceinline__ u2 deq4n2(uint32_t w, h2 d01, h2 d23) {

@@ -526,10 +526,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         return fmaxf(m, sv_[su][i]);
     };
     // both lane halves of a row -> the row's maximum
-    auto row_max = [&](float m) {
-        const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, m), __builtin_bit_cast(unsigned, m), false, false);
-        return fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
-    };
+    auto row_max = [&](float m) { return max_swap32(m); };
     float mloc = NEG_INF;
 #pragma unroll
     for (int idx = 0; idx < 32; ++idx) mloc = mask_max(s_next, tile_of(0) * BN, idx, mloc);

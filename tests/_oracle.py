@@ -54,6 +54,7 @@ def lib():
         L.orc_attn_prep_mrope.argtypes = L.orc_attn_prep.argtypes + [ctypes.POINTER(orc_mrope)]
         L.orc_attn_prep_mrope.restype = ctypes.c_int
         L.orc_a16_quant.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+        L.orc_kv_fill_random.argtypes = [ctypes.POINTER(orc_kv), ctypes.c_int, ctypes.c_int, ctypes.c_uint32]
         L.orc_num_threads.restype = ctypes.c_int
         _lib = L
     return _lib
@@ -189,3 +190,9 @@ def a16_quant(y):
     q = np.zeros(T * ng * 34, np.uint16)
     lib().orc_a16_quant(_p(y), T, n, _p(q))
     return q
+
+
+def kv_fill_random(c, p0, p1, seed):
+    """benchmark fill of positions p0 .. p1 - 1 of one sequence (src/fast/attn.cu:559-581)"""
+    st = c.struct()
+    lib().orc_kv_fill_random(ctypes.byref(st), p0, p1, seed & 0xffffffff)

@@ -77,3 +77,35 @@ def test_paged_dev_and_rows(p1a, kv_type):
     p1a.kv_append_rows(cr, kk, vv, dev(np.array(rows_p, np.int32)), len(rows_p))
     torch.cuda.synchronize()
     assert np.array_equal(pool.dpool.cpu().numpy(), pool.host.pool)
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_fill_random_bytes(p1a, kv_type):
+    """the benchmark fill (the reference's kv_fill_random): contiguous and paged, whole and partial ranges, every byte as
+    the oracle writes it and nothing else touched; a filled cache then decodes like the oracle"""
+    Hq, Hkv, D, psh = 12, 2, 256, 5
+    n = 300
+    host = O.HostKV.contiguous(kv_type, n, Hkv, D)
+    c = p1a.KVCache.contiguous(kv_type, n, Hkv, D)
+    for a, b, seed in [(0, 100, 1), (100, 300, 1), (37, 41, 99), (50, 50, 5)]:
+        O.kv_fill_random(host, a, b, seed)
+        p1a.kv_fill_random(c, a, b, seed)
+    torch.cuda.synchronize()
+    assert np.array_equal(c._keep[0].cpu().numpy(), host.k) and np.array_equal(c._keep[1].cpu().numpy(), host.v)
+    with pytest.raises(p1a.P1AError):
+        p1a.kv_fill_random(c, 0, n + 1, 1)                       # past the end of a contiguous cache
+    lens = [700, 90]
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=8, n_layers=3, layer=2, fill="none")
+    pool.host.pool[:] = 0x33
+    pool.dpool.fill_(0x33)
+    for s, (a, b) in enumerate([(5, 700), (0, 90)]):
+        O.kv_fill_random(pool.host_seq(s), a, b, 0x9e3779b9 * (s + 1))
+        p1a.kv_fill_random(pool.dev_seq(s), a, b, 0x9e3779b9 * (s + 1))
+    torch.cuda.synchronize()
+    assert np.array_equal(pool.dpool.cpu().numpy(), pool.host.pool)
+    from _gpu import check
+    q, _, _, gate = I.qkv(9, 1, 2, Hq, Hkv, D)
+    ref = O.attn_rows(pool.host_seq(0), q, np.array([698, 699], np.int32), Hq, 1 / 16, gate=gate)
+    out = torch.empty((2, Hq, D), device="cuda")
+    p1a.attn_decode(dev(q), pool.dev_seq(0), out, 2, 698, Hq, 1 / 16, gate=dev(gate))
+    check(out.cpu().numpy(), ref, f"decode over a filled cache, type {kv_type}")

@@ -253,3 +253,27 @@ def test_other_shapes_and_refusals(p1a):
         p1a.attn_decode(out, pool.dev_seq(0), out, 1, 5, 5, 0.125)      # Hq not a multiple of Hkv
     torch.cuda.synchronize()
     assert torch.all(out == 7.0)                                        # refused: out untouched
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("low_keys", [(0, 1, 2, 3), (4, 5, 6, 7), (32, 33, 34, 35), tuple(range(0, 16)), tuple(k for k in range(64) if not k & 4)])
+def test_row_maximum_spans_all_lanes(p1a, kv_type, low_keys):
+    """A lane holds four keys of a column and the row maximum is taken across lanes. Keys whose scores sit 2^30 below the
+    rest, placed so that they fill whole lanes (and whole 16-lane rows), must not become the reference of the exponentials:
+    with the maximum of only a part of the lanes P would overflow f16. (The cross-lane exchange once dropped half of
+    its result; softmax does not care which reference it is given until the exponentials leave the f16 range, which
+    RMS-normed random keys never make them do.)"""
+    Hq, Hkv, D, psh, n = 12, 2, 256, 6, 200
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n], seed=81, fill="none")
+    q, k, v, gate = I.qkv(82, n, 2, Hq, Hkv, D)
+    scale = 1.0 / 16.0
+    for hk, h in ((0, 1), (1, 9)):   # one q head of each kv head gets the low keys: k = -c q / |q|^2 scores -c exactly
+        qh = q[0, h]
+        for key in low_keys:
+            k[key, hk] = -(30.0 / (scale * 1.4426950408889634)) * qh / float(qh @ qh)
+    O.kv_append_rows(pool.host_seq(0), k, v, np.arange(n))
+    p1a.kv_append(pool.dev_seq(0), dev(k), dev(v), 0, n)
+    pos = np.array([n - 2, n - 1], np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, scale, gate=gate)
+    out = run_decode(p1a, pool.dev_seq(0), q, 2, n - 2, Hq, scale, gate=gate)
+    check(out, ref, f"low keys {low_keys[:4]}.. type {kv_type}")

@@ -206,3 +206,29 @@ def test_key_split_plan():
     for T, p0, Hq in [(128, 32640, 24), (33, 12000, 24), (300, 777, 12)]:
         ks = p1a.prefill_key_splits(T, p0, Hq)
         assert (p0 + T - 1) // 64 + 1 >= 8 * ks or ks == 1
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("which", ["lower_lane_everywhere", "lower_half", "upper_half", "first_32", "all_but_one"])
+def test_row_maximum_spans_both_lane_halves(p1a, kv_type, which):
+    """the two lanes of a query row each hold 16 keys of a 32-key half tile (keys with bit 2 clear / set) and the row
+    maximum is taken across them: keys scoring 2^30 below the rest and filling one lane's share must not become the
+    reference of the exponentials (P would leave the f16 range)"""
+    Hq, Hkv, D, psh, p0, T = 4, 1, 256, 6, 130, 70
+    n = p0 + T
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n], seed=91, fill="none")
+    q, k, v, gate = I.qkv(92, n, T, Hq, Hkv, D, f16_inputs=True)
+    low = {"lower_lane_everywhere": [x for x in range(n) if not x & 4], "lower_half": [x for x in range(128) if not x & 4], "upper_half": [x for x in range(128) if x & 4],
+           "first_32": list(range(32)), "all_but_one": [x for x in range(128) if x != 77]}[which]
+    # the rows of head 2 share a direction (plus their own noise), and the low keys point against it: every row of that
+    # head scores them about 30 (in powers of two) below zero, the other heads see them as ordinary keys
+    qh = q[0, 2].copy()
+    q[:, 2] = (qh[None, :] + 0.3 * q[:, 2]).astype(np.float16).astype(np.float32)
+    for key in low:
+        k[key, 0] = -(30.0 / (0.1 * 1.4426950408889634)) * qh / float(qh @ qh)
+    O.kv_append_rows(pool.host_seq(0), k, v, np.arange(n))
+    p1a.kv_append(pool.dev_seq(0), dev(k), dev(v), 0, n)
+    pos = p0 + np.arange(T, dtype=np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, 0.1, gate=gate)
+    out = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 0.1, gate=gate)
+    check(out, ref, f"prefill low keys {which} type {kv_type}")
