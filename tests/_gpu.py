@@ -65,13 +65,14 @@ class Pool:
         return self.p1a.KVCache(self.type, self.lens[s], self.Hkv, self.D, dk.data_ptr(), dv.data_ptr(), keep=(dk, dv))
 
 
-def check(out, ref, what=""):
+def check(out, ref, what="", rel_l2_tol=None):
     """max-abs <= 2e-3 (times max|ref| where the reference exceeds 1: the products run on f16 operands, whose error is
     relative - the criterion of the engine's own tests, tests/fast_attn_test.cu:75,217,269 - and outputs above 1 only
     occur for contexts of a few keys) and rel-L2 <= 1e-3"""
     ma, rl = I.errors(out, ref)
     tol = I.MAX_ABS_TOL * max(1.0, float(np.max(np.abs(ref))))
+    rtol = I.REL_L2_TOL if rel_l2_tol is None else rel_l2_tol     # (only tests that craft scores far outside the model's range pass one)
     assert np.all(np.isfinite(out)), what
-    assert ma <= tol and rl <= I.REL_L2_TOL, f"{what}: max_abs={ma:.3e} (tol {tol:.3g}) rel_l2={rl:.3e}"
-    print(f"[parity] {what}: max_abs={ma:.3e} (tol {tol:.3g}) rel_l2={rl:.3e} (tol {I.REL_L2_TOL:g})")   # shown with pytest -s
+    assert ma <= tol and rl <= rtol, f"{what}: max_abs={ma:.3e} (tol {tol:.3g}) rel_l2={rl:.3e} (tol {rtol:g})"
+    print(f"[parity] {what}: max_abs={ma:.3e} (tol {tol:.3g}) rel_l2={rl:.3e} (tol {rtol:g})")   # shown with pytest -s
     return ma, rl

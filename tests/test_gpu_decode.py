@@ -277,3 +277,34 @@ def test_row_maximum_spans_all_lanes(p1a, kv_type, low_keys):
     ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, scale, gate=gate)
     out = run_decode(p1a, pool.dev_seq(0), q, 2, n - 2, Hq, scale, gate=gate)
     check(out, ref, f"low keys {low_keys[:4]}.. type {kv_type}")
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("shape", ["stairs_up", "stairs_down", "spikes"])
+def test_moving_maxima_and_uniform_rows(p1a, kv_type, shape):
+    """scores whose level changes by 2^10 from one 16-key tile to the next (up: every tile moves the reference maximum
+    and rescales the accumulators; down: the exponentials of later tiles underflow; spikes: single keys 2^25 above the
+    rest, scattered over waves and split streams), on top of ordinary random scores; and a query of zeros, whose row
+    must be the plain mean of the visible V rows (closed form)"""
+    Hq, Hkv, D, psh, n = 12, 2, 256, 6, 20000
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n], seed=83, fill="none")
+    q, k, v, gate = I.qkv(84, n, 3, Hq, Hkv, D)
+    scale, l2e = 1.0 / 16.0, 1.4426950408889634
+    tile = np.arange(n) // 16
+    level = {"stairs_up": 10.0 * (tile % 8), "stairs_down": -10.0 * (tile % 8),
+             "spikes": np.where((np.arange(n) * 2654435761 % 4093) < 3, 25.0, 0.0)}[shape]
+    for hk, h in ((0, 2), (1, 7)):
+        qh = q[0, h]
+        k[:, hk] += (level / (scale * l2e))[:, None] * (qh / float(qh @ qh))[None, :]
+    q[2] = 0.0                                                       # the uniform row
+    O.kv_append_rows(pool.host_seq(0), k, v, np.arange(n))
+    p1a.kv_append(pool.dev_seq(0), dev(k), dev(v), 0, n)
+    pos = np.array([n - 3, n - 2, n - 1], np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, scale)
+    out = run_decode(p1a, pool.dev_seq(0), q, 3, n - 3, Hq, scale)
+    # (scores of magnitude 2^5 .. 2^6: the f16 rounding of q and k, 2^-11 relative, moves a score by a few hundredths and
+    # an exponential by a few percent - three times the bound that holds for RMS-normed keys)
+    check(out, ref, f"{shape} type {kv_type}", rel_l2_tol=3e-3)
+    vmean = np.stack([O.kv_read_head(pool.host_seq(0), 1, 0, p, hk) for p in range(n) for hk in range(Hkv)]).reshape(n, Hkv, D).astype(np.float64).mean(0)
+    for h in range(Hq):
+        assert np.abs(out[2, h] - vmean[h // (Hq // Hkv)]).max() < 2e-4, h

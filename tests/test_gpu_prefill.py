@@ -232,3 +232,29 @@ def test_row_maximum_spans_both_lane_halves(p1a, kv_type, which):
     ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, 0.1, gate=gate)
     out = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 0.1, gate=gate)
     check(out, ref, f"prefill low keys {which} type {kv_type}")
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+@pytest.mark.parametrize("shape", ["stairs_up", "stairs_down", "spikes"])
+def test_moving_maxima(p1a, kv_type, shape):
+    """scores whose level changes by 2^10 from one 64-key tile to the next (up: every tile moves the reference maximum of
+    every row and rescales both waves' accumulators; down: later exponentials underflow), or single keys 2^25 above the
+    rest, on top of ordinary random scores; rows of one head share a direction so that the levels hold for all of them"""
+    Hq, Hkv, D, psh, p0, T = 4, 1, 256, 6, 1500, 200
+    n = p0 + T
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n], seed=93, fill="none")
+    q, k, v, gate = I.qkv(94, n, T, Hq, Hkv, D, f16_inputs=True)
+    qh = q[0, 1].copy()
+    q[:, 1] = (qh[None, :] + 0.3 * q[:, 1]).astype(np.float16).astype(np.float32)
+    tile = np.arange(n) // 64
+    level = {"stairs_up": 10.0 * (tile % 6), "stairs_down": -10.0 * (tile % 6),
+             "spikes": np.where((np.arange(n) * 2654435761 % 509) < 3, 25.0, 0.0)}[shape]
+    k[:, 0] += (level / (0.1 * 1.4426950408889634))[:, None] * (qh / float(qh @ qh))[None, :]
+    O.kv_append_rows(pool.host_seq(0), k, v, np.arange(n))
+    p1a.kv_append(pool.dev_seq(0), dev(k), dev(v), 0, n)
+    pos = p0 + np.arange(T, dtype=np.int32)
+    ref = O.attn_rows(pool.host_seq(0), q, pos, Hq, 0.1, gate=gate)
+    out = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 0.1, gate=gate)
+    # (scores of magnitude 2^5 .. 2^6: the f16 rounding of q and k, 2^-11 relative, moves a score by a few hundredths and
+    # an exponential by a few percent - three times the bound that holds for RMS-normed keys)
+    check(out, ref, f"prefill {shape} type {kv_type}", rel_l2_tol=3e-3)
