@@ -107,3 +107,59 @@ def test_config5_append_4096_then_prefill_over_32768(p1a):
     torch.cuda.synchronize()
     ma, rl = I.errors(out.cpu().numpy()[pick], dec.cpu().numpy())
     assert ma < 1e-3 and rl < 5e-4, (ma, rl)
+
+
+@pytest.mark.parametrize("kv_type", [O.KV_Q8_0, O.KV_F16])
+def test_pages_beyond_4_gib(p1a, kv_type):
+    """page bases are 64-bit (the engine keeps one layer's K region under 4 GiB to index it with 32 bits,
+    src/tp_model.cu:3917-3919; this library does not): a pool of > 5 GB whose sequence lives in pages on both sides of the
+    4 GiB line - append, decode, prefill and the benchmark fill all address them, and what they write is, page by page,
+    the oracle's bytes for a contiguous cache"""
+    Hq, Hkv, D, psh, n = 24, 4, 256, 8, 2000
+    ps = 1 << psh
+    rowb = p1a.kv_row_bytes(kv_type, Hkv, D)
+    pstride = 2 * ps * rowb
+    n_pages = (5 << 30) // pstride + 1
+    line = (4 << 30) // pstride                                  # first page that starts beyond 4 GiB
+    pages = [n_pages - 1, line + 90, 3, line + 1, n_pages - 2, line - 1, line + 700, 17]
+    assert len(pages) * ps >= n and pages[0] * pstride > (5 << 30) - pstride
+    tab = dev(np.array(pages, np.int32))
+    pool = torch.empty(n_pages * pstride, dtype=torch.uint8, device="cuda")
+    c = p1a.KVCache.paged(kv_type, Hkv, D, psh, n_pages, tab, len(pages), pool=pool)
+    q, k, v, gate = I.qkv(123, n, 4, Hq, Hkv, D)
+    host = O.HostKV.contiguous(kv_type, len(pages) * ps, Hkv, D)
+    O.kv_append_rows(host, k, v, np.arange(n))
+    p1a.kv_append(c, dev(k), dev(v), 0, n)
+    torch.cuda.synchronize()
+    for g, pg in enumerate(pages):                               # the device pages hold the oracle's rows
+        rows = min(ps, n - g * ps)
+        if rows <= 0:
+            break
+        kd = pool[pg * pstride: pg * pstride + rows * rowb].cpu().numpy()
+        vd = pool[pg * pstride + ps * rowb: pg * pstride + ps * rowb + rows * rowb].cpu().numpy()
+        assert np.array_equal(kd, host.k[g * ps * rowb: (g * ps + rows) * rowb]), g
+        assert np.array_equal(vd, host.v[g * ps * rowb: (g * ps + rows) * rowb]), g
+    pos = np.arange(n - 4, n, dtype=np.int32)
+    ref = O.attn_rows(host, q, pos, Hq, 1 / 16, gate=gate)
+    out = torch.empty((4, Hq, D), device="cuda")
+    p1a.attn_decode(dev(q), c, out, 4, n - 4, Hq, 1 / 16, gate=dev(gate))
+    check(out.cpu().numpy(), ref, f"decode over pages beyond 4 GiB, type {kv_type}")
+    T = 300
+    qp, _, _, gp = I.qkv(124, 1, T, Hq, Hkv, D, f16_inputs=True)
+    refp = O.attn_rows(host, qp, np.arange(n - T, n, dtype=np.int32), Hq, 1 / 16, gate=gp)
+    outp = torch.empty((T, Hq, D), device="cuda")
+    p1a.attn_prefill(dev(qp), c, outp, T, n - T, Hq, 1 / 16, gate=dev(gp))
+    check(outp.cpu().numpy(), refp, f"prefill over pages beyond 4 GiB, type {kv_type}")
+    O.kv_fill_random(host, 100, n, 77)                           # (paged fill = page by page with the page's seed:
+    hp = O.HostKV.paged(kv_type, Hkv, D, psh, len(pages), np.arange(len(pages), dtype=np.int32), len(pages))   # a compact host twin)
+    hp.pool[:] = 0
+    O.kv_append_rows(hp, k, v, np.arange(n))
+    O.kv_fill_random(hp, 100, n, 77)
+    p1a.kv_fill_random(c, 100, n, 77)
+    torch.cuda.synchronize()
+    for g, pg in enumerate(pages):
+        got = pool[pg * pstride: (pg + 1) * pstride].cpu().numpy()
+        rows = max(0, min(ps, n - g * ps))
+        want = hp.pool[g * pstride: (g + 1) * pstride]
+        assert np.array_equal(got[: rows * rowb], want[: rows * rowb]), g
+        assert np.array_equal(got[ps * rowb: ps * rowb + rows * rowb], want[ps * rowb: ps * rowb + rows * rowb]), g
