@@ -134,6 +134,41 @@ static void test_type(uint32_t type, hipStream_t s) {
         auto a = bytes_of(o1, (size_t) T * Hq * D * 4), b = bytes_of(o2, (size_t) T * Hq * D * 4);
         check("attn_prefill T=200 p0=1300 paged vs contiguous", a1 && a2 && !memcmp(a.data(), b.data(), a.size()));
     }
+    {   // attn_fold on a short chunk over a long context (the library splits it over the keys): with the scratch of
+        // attn_fold_scratch_bytes, with a scratch that is too small and through attn_prefill - one result, bit for bit
+        const int sq = 1, T = 100, p0 = len[sq] - T;
+        const size_t nb = F::attn_fold_scratch_bytes(T, Hkv, 2048, 8, p0);
+        void * scr; CK(hipMalloc(&scr, nb)); CK(hipMemset(scr, 0xff, nb));
+        const bool a1 = F::attn_prefill(q, cc[sq], o1, T, p0, Hq, scale, s);
+        CK(hipStreamSynchronize(s));
+        auto a = bytes_of(o1, (size_t) T * Hq * D * 4);
+        const bool a2 = F::attn_fold(q, paged(sq), o2, T, p0, Hq, scale, scr, nb, s);
+        CK(hipStreamSynchronize(s));
+        auto b = bytes_of(o2, (size_t) T * Hq * D * 4);
+        const bool a3 = F::attn_fold(q, cc[sq], o2, T, p0, Hq, scale, scr, 4096, s);
+        CK(hipStreamSynchronize(s));
+        auto c3 = bytes_of(o2, (size_t) T * Hq * D * 4);
+        printf("    (%d key splits) ", p1a_attn_prefill_key_splits(T, p0, Hq));
+        check("attn_fold (scratch, paged) vs attn_fold (small scratch) vs attn_prefill", a1 && a2 && a3 && p1a_attn_prefill_key_splits(T, p0, Hq) > 1 &&
+              !memcmp(a.data(), b.data(), a.size()) && !memcmp(a.data(), c3.data(), a.size()));
+        CK(hipFree(scr));
+    }
+    {   // kv_fill_random: a function of (position range, seed) alone, touching nothing else
+        F::kv_cache f1 = F::kv_alloc(type, 512, Hkv, D), f2 = F::kv_alloc(type, 512, Hkv, D);
+        F::kv_fill_random(f1, 10, 300, 42u, s);
+        F::kv_fill_random(f2, 10, 150, 42u, s);
+        F::kv_fill_random(f2, 150, 300, 42u, s);
+        CK(hipStreamSynchronize(s));
+        auto a = bytes_of(f1.k, 512 * rowb), b = bytes_of(f2.k, 512 * rowb), va = bytes_of(f1.v, 512 * rowb), vb = bytes_of(f2.v, 512 * rowb);
+        bool ok = a == b && va == vb;
+        for (size_t i = 0; i < 10 * rowb; ++i) ok = ok && a[i] == 0;
+        for (size_t i = 300 * rowb; i < 512 * rowb; ++i) ok = ok && a[i] == 0 && va[i] == 0;
+        F::kv_fill_random(f2, 10, 300, 43u, s);
+        CK(hipStreamSynchronize(s));
+        ok = ok && bytes_of(f2.k, 512 * rowb) != a;
+        check("kv_fill_random: ranges add up, other rows untouched, seed matters", ok);
+        F::kv_free(f1); F::kv_free(f2);
+    }
     {   // attn_prep: host positions on the contiguous cache vs device positions through the page table (one sequence)
         const int sq = 2, T = 4, p0 = len[sq] - T, n_rot = 64;
         float * qg = dev_rand((size_t) T * Hq * 2 * D, 1.0f), * kk = dev_rand((size_t) T * Hkv * D, 1.0f), * vv = dev_rand((size_t) T * Hkv * D, 1.0f);
