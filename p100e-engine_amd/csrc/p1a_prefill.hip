@@ -280,11 +280,19 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     // ---- Q^T operands (B: k = 16 dims per step, n = query row): lane (row c, half g) holds dims 16 ks + 8 g .. + 7 ----
     h8 qf[C::NKS];
     {
+        // (all the loads first, then the conversions: a load that is waited for before the next one is asked for costs a
+        // memory round trip each - 16 of them in a row were most of what a workgroup spent outside its key loop)
         const float * qr = P.q + ((size_t) (live ? my_tok : 0) * P.Hq + h) * D;
+        float4 qa[C::NKS], qb[C::NKS];
 #pragma unroll
         for (int ks = 0; ks < C::NKS; ++ks) {
-            float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
-            if (live) { a = *reinterpret_cast<const float4 *>(qr + 16 * ks + 8 * g); b = *reinterpret_cast<const float4 *>(qr + 16 * ks + 8 * g + 4); }
+            qa[ks] = make_float4(0.f, 0.f, 0.f, 0.f);
+            qb[ks] = qa[ks];
+            if (live) { qa[ks] = *reinterpret_cast<const float4 *>(qr + 16 * ks + 8 * g); qb[ks] = *reinterpret_cast<const float4 *>(qr + 16 * ks + 8 * g + 4); }
+        }
+#pragma unroll
+        for (int ks = 0; ks < C::NKS; ++ks) {
+            const float4 a = qa[ks], b = qb[ks];
             const float s = P.qscale;
             qf[ks] = h8{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s),
                         (half_t) (b.x * s), (half_t) (b.y * s), (half_t) (b.z * s), (half_t) (b.w * s)};
@@ -733,6 +741,15 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         const float inv = 1.0f / (r ? l_par : ol[0]);
         float * orow = P.out + ((size_t) tok * P.Hq + h) * D;
         const float * grow = P.gate ? P.gate + ((size_t) tok * P.Hq + h) * D : nullptr;
+        // (the gate values of the row's half are all asked for before the first is used: one memory round trip, not one per
+        // 16 bytes)
+        f4 gt[HD][4];
+        if (grow) {
+#pragma unroll
+            for (int dt = 0; dt < HD; ++dt)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) gt[dt][q4] = *reinterpret_cast<const f4 *>(grow + 32 * (dh * HD + dt) + 8 * q4 + 4 * g);
+        }
 #pragma unroll
         for (int dt = 0; dt < HD; ++dt)
 #pragma unroll
@@ -740,9 +757,8 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                 const int d0 = 32 * (dh * HD + dt) + 8 * q4 + 4 * g;
                 f4 rr = {o[r][dt][4 * q4] * inv, o[r][dt][4 * q4 + 1] * inv, o[r][dt][4 * q4 + 2] * inv, o[r][dt][4 * q4 + 3] * inv};
                 if (grow) {
-                    const f4 gt = *reinterpret_cast<const f4 *>(grow + d0);
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) rr[x] *= 1.0f / (1.0f + expf(-gt[x]));
+                    for (int x = 0; x < 4; ++x) rr[x] *= 1.0f / (1.0f + expf(-gt[dt][q4][x]));
                 }
                 *reinterpret_cast<f4 *>(orow + d0) = rr;
             }
