@@ -279,11 +279,13 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
 
     // ---- Q^T operands (B: k = 16 dims per step, n = query row): lane (row c, half g) holds dims 16 ks + 8 g .. + 7 ----
     h8 qf[C::NKS];
-    {
-        // (all the loads first, then the conversions: a load that is waited for before the next one is asked for costs a
-        // memory round trip each - 16 of them in a row were most of what a workgroup spent outside its key loop)
-        const float * qr = P.q + ((size_t) (live ? my_tok : 0) * P.Hq + h) * D;
+    // (all the loads first, then the conversions: a load that is waited for before the next one is asked for costs a
+    // memory round trip each - 16 of them in a row were most of what a workgroup spent outside its key loop. With
+    // LDS-direct tiles the rows are asked for right behind the first tiles (the compiler drains its own loads in front of
+    // hand-issued ones, so asking earlier would put the two latencies in a row): one latency, not two.)
+    auto load_q = [&]() {
         float4 qa[C::NKS], qb[C::NKS];
+        const float * qr = P.q + ((size_t) (live ? my_tok : 0) * P.Hq + h) * D;
 #pragma unroll
         for (int ks = 0; ks < C::NKS; ++ks) {
             qa[ks] = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -300,7 +302,8 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             // the vector registers are left to the tiles in flight
             asm volatile("" : "+a"(qf[ks]));
         }
-    }
+    };
+    if constexpr (!DMA) load_q();
 
     // Waves pair up for O^T: the pair (w, w ^ 1) shares its 64 query rows, each wave accumulating HALF the dims
     // (tiles HD * (w & 1) ..) for ALL 64 rows: a V^T fragment read from LDS then feeds two MFMAs (own rows, partner's
@@ -507,6 +510,7 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         for (int j = 0; j < 8; ++j) dma_block(P.vc, b0, lds + L::KT_B, L::VB, j);
 #pragma unroll
         for (int j = 0; j < 8; ++j) dma_block(P.kc, gb_prev, lds + L::STAGE_B, L::KB, j);
+        load_q();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         zero_v_tail(tile_of(0), lds + L::KT_B);
     } else {
@@ -734,34 +738,38 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         return;
     }
     const float l_par = ax_par[c];
+    // (the gate values of both row blocks are asked for before the first is used: one memory round trip, not one per 16
+    // bytes or per block)
+    f4 gt[2][HD][4];
+    if (P.gate) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r) {
+            const int tok = tok0 + 32 * (r ? wave ^ 1 : wave) + c;
+            const float * grow = P.gate + ((size_t) min(tok, P.T - 1) * P.Hq + h) * D;
+#pragma unroll
+            for (int dt = 0; dt < HD; ++dt)
+#pragma unroll
+                for (int q4 = 0; q4 < 4; ++q4) gt[r][dt][q4] = *reinterpret_cast<const f4 *>(grow + 32 * (dh * HD + dt) + 8 * q4 + 4 * g);
+        }
+    }
 #pragma unroll
     for (int r = 0; r < 2; ++r) {
         const int tok = tok0 + 32 * (r ? wave ^ 1 : wave) + c;
         if (tok >= P.T) continue;
         const float inv = 1.0f / (r ? l_par : ol[0]);
         float * orow = P.out + ((size_t) tok * P.Hq + h) * D;
-        const float * grow = P.gate ? P.gate + ((size_t) tok * P.Hq + h) * D : nullptr;
-        // (the gate values of the row's half are all asked for before the first is used: one memory round trip, not one per
-        // 16 bytes)
-        f4 gt[HD][4];
-        if (grow) {
-#pragma unroll
-            for (int dt = 0; dt < HD; ++dt)
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) gt[dt][q4] = *reinterpret_cast<const f4 *>(grow + 32 * (dh * HD + dt) + 8 * q4 + 4 * g);
-        }
 #pragma unroll
         for (int dt = 0; dt < HD; ++dt)
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {
                 const int d0 = 32 * (dh * HD + dt) + 8 * q4 + 4 * g;
                 f4 rr = {o[r][dt][4 * q4] * inv, o[r][dt][4 * q4 + 1] * inv, o[r][dt][4 * q4 + 2] * inv, o[r][dt][4 * q4 + 3] * inv};
-                if (grow) {
+                if (P.gate) {
                     // sigmoid through the hardware exponential and reciprocal (each within an ulp or two; exact at g = 0): the
                     // library's full-range expf and IEEE division are some twenty instructions per value, 128 values per lane
 #pragma unroll
                     for (int x = 0; x < 4; ++x)
-                        rr[x] *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gt[dt][q4][x]));
+                        rr[x] *= __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * gt[r][dt][q4][x]));
                 }
                 *reinterpret_cast<f4 *>(orow + d0) = rr;
             }
