@@ -196,3 +196,9 @@ def kv_fill_random(c, p0, p1, seed):
     """benchmark fill of positions p0 .. p1 - 1 of one sequence (src/fast/attn.cu:559-581)"""
     st = c.struct()
     lib().orc_kv_fill_random(ctypes.byref(st), p0, p1, seed & 0xffffffff)
+
+
+def gate(x, g):
+    """in place: x *= 1 / (1 + exp(-g)) (src/kernels.cu:85-88); x, g float32 arrays of one size"""
+    assert x.dtype == np.float32 and g.dtype == np.float32 and x.size == g.size and x.flags.c_contiguous and g.flags.c_contiguous
+    lib().orc_gate(x.ctypes.data, g.ctypes.data, x.size)

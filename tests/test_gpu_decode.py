@@ -308,3 +308,29 @@ def test_moving_maxima_and_uniform_rows(p1a, kv_type, shape):
     vmean = np.stack([O.kv_read_head(pool.host_seq(0), 1, 0, p, hk) for p in range(n) for hk in range(Hkv)]).reshape(n, Hkv, D).astype(np.float64).mean(0)
     for h in range(Hq):
         assert np.abs(out[2, h] - vmean[h // (Hq // Hkv)]).max() < 2e-4, h
+
+
+def test_standalone_gate_equals_the_fused_one(p1a):
+    """sigmoid_mul (the engine's k::sigmoid_mul launch behind attention) on an ungated decode == the decode with the gate
+    fused into its merge, bit for bit (one formula); and against the oracle's gate, with the closed form g = 0 -> x 0.5"""
+    Hq, Hkv, D, n = 12, 2, 256, 900
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, 6, [n], seed=97)
+    q, _, _, gate = I.qkv(98, 1, 3, Hq, Hkv, D)
+    gate[0, :64] = 0.0
+    gate[1, :8] = [-200.0, 200.0, -90.0, 90.0, -30.0, 30.0, -1e-8, 1e-8]      # saturation and the flat middle
+    dq, dg = dev(q), dev(gate)
+    plain = torch.empty((3, Hq, D), device="cuda")
+    fused = torch.empty((3, Hq, D), device="cuda")
+    p1a.attn_decode(dq, pool.dev_seq(0), plain, 3, n - 3, Hq, 1 / 16)
+    p1a.attn_decode(dq, pool.dev_seq(0), fused, 3, n - 3, Hq, 1 / 16, gate=dg)
+    ungated = plain.cpu().numpy().copy()
+    p1a.sigmoid_mul(plain, dg)
+    torch.cuda.synchronize()
+    assert torch.equal(plain, fused)
+    want = ungated.reshape(3, -1).copy()
+    O.gate(want, gate)
+    got = plain.cpu().numpy().reshape(3, -1)
+    assert np.all(np.isfinite(got))
+    assert np.abs(got - want).max() <= 1e-6 * max(1.0, np.abs(want).max())
+    assert np.array_equal(got[0, :64], 0.5 * ungated.reshape(3, -1)[0, :64])
+    assert np.all(got[1, [0]] == 0.0 * ungated.reshape(3, -1)[1, [0]])       # sigmoid(-200) = 0: expf overflows to inf, 1 / inf = 0
