@@ -103,3 +103,45 @@ def test_growth_during_capture_is_refused_and_knobs(p1a):
     p1a.attn_decode(dq, c, out, 2, n - 2, Hq, 1 / 16, gate=dg)
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy(), base)
+
+
+def test_two_streams_and_two_host_threads(p1a):
+    """calls on different streams of one device may overlap (the split buffers belong to a (device, stream) pair, the table of
+    pairs is mutex-protected): two host threads, each on its own stream, run decode and key-split prefill calls over their
+    own sequences at the same time, many times; every result equals the one computed alone"""
+    import threading
+    Hq, Hkv, D, psh = 12, 2, 256, 6
+    lens = [6000, 4500]
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, psh, lens, seed=115)
+    work = []
+    for sq, n in enumerate(lens):
+        q, _, _, gate = I.qkv(116 + sq, 1, 4, Hq, Hkv, D)
+        qp, _, _, gp = I.qkv(118 + sq, 1, 100, Hq, Hkv, D, f16_inputs=True)
+        work.append(dict(c=pool.dev_seq(sq), n=n, q=dev(q), g=dev(gate), qp=dev(qp), gp=dev(gp)))
+    assert p1a.prefill_key_splits(100, lens[0] - 100, Hq) > 1
+    def once(w, out, outp):
+        p1a.attn_decode(w["q"], w["c"], out, 4, w["n"] - 4, Hq, 1 / 16, gate=w["g"])
+        p1a.attn_prefill(w["qp"], w["c"], outp, 100, w["n"] - 100, Hq, 1 / 16, gate=w["gp"])
+    alone = []
+    for w in work:
+        out, outp = torch.zeros((4, Hq, D), device="cuda"), torch.zeros((100, Hq, D), device="cuda")
+        once(w, out, outp)
+        torch.cuda.synchronize()
+        alone.append((out.clone(), outp.clone()))
+    bad = []
+    def run(i):
+        s = torch.cuda.Stream()
+        w = work[i]
+        with torch.cuda.stream(s):
+            for rep in range(40):
+                out, outp = torch.zeros((4, Hq, D), device="cuda"), torch.zeros((100, Hq, D), device="cuda")
+                once(w, out, outp)
+                if rep % 8 == 7:
+                    s.synchronize()
+                    if not (torch.equal(out, alone[i][0]) and torch.equal(outp, alone[i][1])):
+                        bad.append((i, rep))
+            s.synchronize()
+    th = [threading.Thread(target=run, args=(i,)) for i in range(2)]
+    for t in th: t.start()
+    for t in th: t.join()
+    assert not bad, bad
