@@ -258,3 +258,26 @@ def test_moving_maxima(p1a, kv_type, shape):
     # (scores of magnitude 2^5 .. 2^6: the f16 rounding of q and k, 2^-11 relative, moves a score by a few hundredths and
     # an exponential by a few percent - three times the bound that holds for RMS-normed keys)
     check(out, ref, f"prefill {shape} type {kv_type}", rel_l2_tol=3e-3)
+
+
+@pytest.mark.parametrize("kv_type", TYPES)
+def test_sequence_selected_through_the_row_table(p1a, kv_type):
+    """one sequence per prefill call: its page table is pt + rtab[0] when the descriptor carries a row table (how a batched
+    descriptor of the engine names a slot), the same bits as the descriptor whose pt already points at the slot's row; the
+    benchmark fill follows the same rule"""
+    Hq, Hkv, D, psh = 12, 2, 256, 5
+    lens = [300, 700, 90]
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=131)
+    sq, T = 1, 180
+    p0 = lens[sq] - T
+    q, _, _, gate = I.qkv(132, 1, T, Hq, Hkv, D, f16_inputs=True)
+    a = run_prefill(p1a, pool.dev_seq(sq), q, T, p0, Hq, 1 / 16, gate=gate)
+    rt = dev(np.array([sq * pool.maxp, 0, 0], np.int32))
+    b = run_prefill(p1a, pool.devkv.with_rows(rt), q, T, p0, Hq, 1 / 16, gate=gate)
+    assert np.array_equal(a, b)
+    ref = O.attn_rows(pool.host_seq(sq), q, p0 + np.arange(T, dtype=np.int32), Hq, 1 / 16, gate=gate)
+    check(b, ref, f"prefill through the row table, type {kv_type}")
+    O.kv_fill_random(pool.host.view(rtab=np.array([sq * pool.maxp], np.int32)), 10, 600, 5)
+    p1a.kv_fill_random(pool.devkv.with_rows(rt), 10, 600, 5)
+    torch.cuda.synchronize()
+    assert np.array_equal(pool.dpool.cpu().numpy(), pool.host.pool)
