@@ -42,15 +42,25 @@ def test_decode_random_case(p1a, case):
     T = nseq * rps
     q, _, _, gate = I.qkv(9200 + case, 1, T, Hq, Hkv, D)
     pos = np.array([lens[s] - rps + t for s in range(nseq) for t in range(rps)], np.int32)
+    scattered = case % 2 == 1
+    if scattered:   # the rows of a group at any positions of their sequence, in any order (they still share one KV read)
+        pos = np.array([int(g.integers(0, lens[s])) for s in range(nseq) for _ in range(rps)], np.int32)
     rtab = np.array([s * pool.maxp for s in range(nseq) for _ in range(rps)], np.int32)
     ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, scale, gate=gate if use_gate else None)
     out = torch.full((T, Hq, D), float("nan"), device="cuda")
-    what = f"decode case {case}: type {kv_type} {Hq}/{Hkv}/{D} psh {psh} lens {lens} rows/seq {rps} gate {use_gate}"
+    what = f"decode case {case}: type {kv_type} {Hq}/{Hkv}/{D} psh {psh} lens {lens} rows/seq {rps} gate {use_gate} pos {pos.tolist()}"
     print(what, flush=True)
     p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, T, dev(pos), Hq, scale,
                          gate=dev(gate) if use_gate else None, rows_per_seq=rps)
     torch.cuda.synchronize()
     check(out.cpu().numpy(), ref, what)
+    if scattered:   # every row alone at its position: the same bits as in the batch
+        for t in range(min(T, 6)):
+            one = torch.full((1, Hq, D), float("nan"), device="cuda")
+            p1a.attn_decode(dev(q[t:t + 1]), pool.dev_seq(t // rps), one, 1, int(pos[t]), Hq, scale, gate=dev(gate[t:t + 1]) if use_gate else None)
+            torch.cuda.synchronize()
+            assert torch.equal(one[0], out[t]), (what, t)
+        return
     # the first sequence alone, through the one-sequence entry (host position): the same bits as its rows in the batch
     one = torch.full((rps, Hq, D), float("nan"), device="cuda")
     p1a.attn_decode(dev(q[:rps]), pool.dev_seq(0), one, rps, lens[0] - rps, Hq, scale, gate=dev(gate[:rps]) if use_gate else None)
