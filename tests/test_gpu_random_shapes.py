@@ -139,3 +139,60 @@ def test_append_random_case(p1a, case):
             a += m
     torch.cuda.synchronize()
     assert np.array_equal(pool.dpool.cpu().numpy(), pool.host.pool), what
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_prep_random_case(p1a, case):
+    """attn_prep (q | gate split, per-head RMS norm * weight, NEOX rotation of the first n_rot dims, quantizing KV write)
+    over random shapes, rotary widths, row strides, positions up to a million, host-position and device-position mode, with
+    and without interleaved M-RoPE: gate and V bytes exact, q within one ulp (two double-precision trigonometry libraries),
+    K bytes equal but for the few codes a last-bit difference of the rotated value moves"""
+    g = I.rng(9300 + case)
+    kv_type = TYPES[int(g.integers(3))]
+    D = int(g.choice([64, 128, 256]))
+    Hkv = int(g.choice([1, 2, 4]))
+    Hq = Hkv * int(g.choice([1, 2, 6]))
+    n_rot = int(g.choice([0, 8, 32, 64, D]))
+    T = int(g.integers(1, 24))
+    base = float(g.choice([1e4, 1e6, 1e7]))
+    dev_pos = bool(g.integers(2))
+    far = int(g.choice([0, 1000, 250000, 1000000]))            # rotary positions far from the cache rows (M-RoPE style offsets aside)
+    n_ctx = 64
+    rows = g.permutation(n_ctx)[:T].astype(np.int32) if dev_pos else (int(g.integers(0, n_ctx - T)) + np.arange(T)).astype(np.int32)
+    qg = I.normal(g, (T, Hq, 2 * D)); k = I.normal(g, (T, Hkv, D)) * 1.3; v = I.normal(g, (T, Hkv, D))
+    qn = (1.0 + 0.1 * I.normal(g, (D,))).astype(np.float32); kn = (1.0 + 0.1 * I.normal(g, (D,))).astype(np.float32)
+    use_mr = bool(g.integers(2)) and n_rot >= 8
+    mr_host = mr_dev = None
+    if use_mr:
+        npairs = n_rot // 2
+        s0 = int(g.integers(0, npairs + 1)); s1 = int(g.integers(0, npairs - s0 + 1)); s2 = int(g.integers(0, npairs - s0 - s1 + 1))
+        sect = npairs if g.integers(2) else s0 + s1 + s2 + int(g.integers(0, 3))
+        sect = max(sect, 1)
+        stride = T + int(g.integers(0, 4))
+        mp = np.zeros((3, stride), np.int32)
+        mp[:, :T] = far + g.integers(0, 5000, size=(3, T))
+        mr_host, mr_dev = (mp, (s0, s1, s2), sect), (dev(mp), stride, (s0, s1, s2), sect)
+    pos = rows if (dev_pos or not far) and not use_mr else rows          # cache rows = rotary positions unless M-RoPE gives its own
+    ldq, ldk, ldv = Hq * 2 * D + 4 * int(g.integers(0, 3)), Hkv * D + 4 * int(g.integers(0, 3)), Hkv * D + 4 * int(g.integers(0, 3))
+    def strided(a, ld):
+        buf = np.full((T, ld), 3.0, np.float32)
+        buf[:, : a[0].size] = a.reshape(T, -1)
+        return buf
+    what = f"prep case {case}: type {kv_type} {Hq}/{Hkv}/{D} n_rot {n_rot} T {T} base {base:g} dev_pos {dev_pos} mrope {mr_host[1:] if use_mr else None}"
+    print(what, flush=True)
+    host = O.HostKV.contiguous(kv_type, n_ctx, Hkv, D)
+    p0 = -1 if dev_pos else int(rows[0])
+    q_ref, gate_ref = O.attn_prep(host, qg, k, v, qn, kn, pos, p0, Hq, n_rot, base, 1e-6, mrope=mr_host)
+    c = p1a.KVCache.contiguous(kv_type, n_ctx, Hkv, D)
+    q = torch.zeros((T, Hq, D), device="cuda"); gate = torch.zeros((T, Hq * D), device="cuda")
+    p1a.attn_prep(dev(strided(qg, ldq)), dev(strided(k, ldk)), dev(strided(v, ldv)), dev(qn), dev(kn), dev(pos), q, gate, c, p0, T, Hq,
+                  n_rot, base, 1e-6, ldq=ldq, ldk=ldk, ldv=ldv, mrope=mr_dev)
+    torch.cuda.synchronize()
+    assert np.array_equal(gate.cpu().numpy(), gate_ref), what
+    qd = q.cpu().numpy()
+    ia, ib = qd.view(np.int32).astype(np.int64), q_ref.view(np.int32).astype(np.int64)
+    ia, ib = np.where(ia < 0, -(ia & 0x7fffffff), ia), np.where(ib < 0, -(ib & 0x7fffffff), ib)
+    assert np.abs(ia - ib).max() <= 1, (what, int(np.abs(ia - ib).max()))
+    assert np.array_equal(c._keep[1].cpu().numpy(), host.v), what
+    kd = c._keep[0].cpu().numpy()
+    assert np.count_nonzero(kd != host.k) <= max(4, kd.size // 5000), (what, int(np.count_nonzero(kd != host.k)))
