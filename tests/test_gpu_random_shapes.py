@@ -54,6 +54,14 @@ def test_decode_random_case(p1a, case):
                          gate=dev(gate) if use_gate else None, rows_per_seq=rps)
     torch.cuda.synchronize()
     check(out.cpu().numpy(), ref, what)
+    if case % 4 == 0:   # the same call with the a16 activation buffer of its (gated) rows: same output bits, the oracle's buffer
+        out2 = torch.full((T, Hq, D), float("nan"), device="cuda")
+        qb = torch.zeros(p1a.a16_bytes(T, Hq * D) // 2, dtype=torch.int16, device="cuda")
+        p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out2, T, dev(pos), Hq, scale,
+                             gate=dev(gate) if use_gate else None, rows_per_seq=rps, qbuf=qb)
+        torch.cuda.synchronize()
+        assert torch.equal(out, out2), what
+        assert np.array_equal(qb.cpu().numpy().view(np.uint16), O.a16_quant(out2.cpu().numpy().reshape(T, Hq * D))), what
     if scattered:   # every row alone at its position: the same bits as in the batch
         for t in range(min(T, 6)):
             one = torch.full((1, Hq, D), float("nan"), device="cuda")
