@@ -50,9 +50,13 @@ def build_pool(p1a, torch, kv_type, Hq, Hkv, D, psh, n_ctx, n_seq, seed, lens=No
     return kv, ppseq
 
 
-def time_graph(torch, stream, fn_list, warmup):
-    """capture the calls of fn_list into one graph on `stream`, replay `warmup` times, then time one replay with
-    events recorded on that same stream. Returns seconds per call."""
+REPLAYS = 7   # timed replays of a captured graph; the median is reported
+
+
+def time_graph(torch, stream, fn_list, warmup, replays=REPLAYS, all_samples=False):
+    """capture the calls of fn_list into one graph on `stream`, run `warmup` untimed calls (whole replays: at least one),
+    then time `replays` replays, each bracketed by a synchronize and by events recorded on that same stream. Returns the
+    MEDIAN seconds per call (and, on request, every sample)."""
     with torch.cuda.stream(stream):
         for f in fn_list[:2]:
             f()
@@ -61,33 +65,43 @@ def time_graph(torch, stream, fn_list, warmup):
         with torch.cuda.graph(g, stream=stream):
             for f in fn_list:
                 f()
-        for _ in range(max(1, warmup)):
+        for _ in range(max(1, -(-warmup // len(fn_list)))):
             g.replay()
         stream.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        e0.record(stream)
-        g.replay()
-        e1.record(stream)
-        e1.synchronize()
-        torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / len(fn_list)
+        samples = []
+        for _ in range(replays):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record(stream)
+            g.replay()
+            e1.record(stream)
+            e1.synchronize()
+            torch.cuda.synchronize()
+            samples.append(e0.elapsed_time(e1) * 1e-3 / len(fn_list))
+    samples.sort()
+    med = samples[len(samples) // 2]
+    return (med, samples) if all_samples else med
 
 
-def time_eager(torch, fn, reps, warmup=2):
+def time_eager(torch, fn, reps, warmup=2, group=1):
+    """median over `reps` samples, each `group` back-to-back calls event-timed on the current stream; seconds per call"""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
+    samples = []
     for _ in range(reps):
-        fn()
-    e1.record()
-    e1.synchronize()
-    return e0.elapsed_time(e1) * 1e-3 / reps
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(group):
+            fn()
+        e1.record()
+        e1.synchronize()
+        samples.append(e0.elapsed_time(e1) * 1e-3 / group)
+    samples.sort()
+    return samples[len(samples) // 2]
 
 
-def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
+def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
     """secondary measurements: the other baseline configs at full size (reported, not the headline value)"""
     import math
     ex = {}
@@ -114,18 +128,29 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale):
     ex["prefill_TFLOPs"] = round(flop / sec / 1e12, 1)
     ex["prefill_frac_of_f16_mfma_peak"] = round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)
     ex["prefill_scratch_MB"] = round(scr.numel() / 1e6, 1)
+    top["roofline_prefill"] = {
+        "bound": "mfma", "achieved": round(flop / sec / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "prefill_k<f16, 256, grouped, lds-direct>",
+        "call_ms": round(sec * 1e3, 4),
+        "note": "configs[4]: T = 4096 after 28672 tokens, q8_0, fused gate; flops = 4 D Hq (p0 T + T (T + 1) / 2); time = the "
+                "whole p1a_attn_prefill call with caller scratch (the convert-once pass of about 40 us included), median of 5"}
+    out_scr = out.clone()
     sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=5)
     ex["prefill_no_scratch_ms"] = round(sec * 1e3, 4)
-    del scr
+    ex["prefill_no_scratch_frac_of_f16_mfma_peak"] = round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)
+    ex["prefill_scratch_equals_no_scratch_bits"] = bool(torch.equal(out, out_scr))
+    del scr, out_scr
+    if cpu:
+        top["cpu_prefill"] = cpu_prefill(torch, kv, ppseq, q, gate, out, p0, T, Hq, Hkv, D, psh, scale)
     # a short last chunk over the same context: its keys are split over several workgroups per (token block, head)
     Ts, p0s = 128, p0 + T - 128
     scr = torch.empty(p1a.prefill_scratch_bytes(Ts, p0s, Hq, Hkv, D), dtype=torch.uint8, device="cuda")
-    sec = time_eager(torch, lambda: p1a.attn_prefill(q[:Ts], c, out[:Ts], Ts, p0s, Hq, scale, gate=gate[:Ts], scratch=scr), reps=10)
+    sec = time_eager(torch, lambda: p1a.attn_prefill(q[:Ts], c, out[:Ts], Ts, p0s, Hq, scale, gate=gate[:Ts], scratch=scr), reps=5, group=10)
     ex["prefill_T128_p32640_q8_0_us"] = round(sec * 1e6, 1)
     ex["prefill_T128_key_splits"] = p1a.prefill_key_splits(Ts, p0s, Hq)
     ex["prefill_T128_TFLOPs"] = round(4.0 * D * Hq * (p0s * Ts + Ts * (Ts + 1) / 2) / sec / 1e12, 1)
     del scr
-    sec = time_eager(torch, lambda: p1a.kv_append(c, kc, vc, p0, T), reps=20)
+    sec = time_eager(torch, lambda: p1a.kv_append(c, kc, vc, p0, T), reps=5, group=20)
     ab = 2 * T * Hkv * D * 4 + 2 * T * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
     ex["append_T4096_q8_0_us"] = round(sec * 1e6, 2)
     ex["append_GBs"] = round(ab / sec / 1e9, 1)
@@ -256,27 +281,81 @@ def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, step
             "mtp_loop": f"{n_seq} sequences x (1 + 3 drafts), q4_0, ~{ctx} tokens each, prep + decode + accept/rollback, wall clock"}
 
 
-def cpu_baseline(Hq, Hkv, D, n_ctx, seed):
-    """The CPU oracle (fp32 restatement of the reference's attention kernel) on a bounded sample of the same
-    workload: one query row over a q8_0 cache of n_ctx tokens, repeated for about 10 s."""
+def host_cpu():
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return model, os.cpu_count()
+
+
+def host_view(torch, kv, ppseq, slot, Hkv, D, psh, kv_type):
+    """the oracle's view of one sequence of a device pool: the pool's bytes and its page table copied to the host"""
+    import numpy as np
+    import _oracle as O
+    pool = kv.pool.cpu().numpy()
+    tabs = kv.pt.cpu().numpy() if hasattr(kv.pt, "cpu") else kv._keep[1].cpu().numpy()
+    n_pages = pool.size // kv.pstride
+    h = O.HostKV.paged(kv_type, Hkv, D, psh, n_pages, tabs, ppseq, pool=pool)
+    return h.view(pt=np.ascontiguousarray(tabs[slot * ppseq:(slot + 1) * ppseq]))
+
+
+def cpu_baseline(torch, kv, ppseq, slot, q, gate, out_gpu, Hq, Hkv, D, psh, n_ctx, scale):
+    """The CPU oracle (fp32 restatement of the reference's attention kernel, OpenMP over heads) on a bounded sample of
+    the same workload: the decode step the GPU timed last - same pool bytes, same page table, same q and gate - repeated
+    for about 10 s; its result is the check of the GPU's timed output."""
     import numpy as np
     import _inputs as I
     import _oracle as O
-    q, k, v, gate = I.qkv(seed, n_ctx, 1, Hq, Hkv, D)
-    c = O.HostKV.contiguous(O.KV_Q8_0, n_ctx, Hkv, D)
-    O.kv_append_rows(c, k, v, np.arange(n_ctx))
+    hv = host_view(torch, kv, ppseq, slot, Hkv, D, psh, O.KV_Q8_0)
+    hq, hg = q.cpu().numpy(), gate.cpu().numpy()
     pos = np.array([n_ctx - 1], np.int32)
-    O.attn_rows(c, q, pos, Hq, 1.0 / 16, gate=gate)
+    ref = O.attn_rows(hv, hq, pos, Hq, scale, gate=hg)
     reps, t0 = 0, time.perf_counter()
     while True:
-        out = O.attn_rows(c, q, pos, Hq, 1.0 / 16, gate=gate)
+        O.attn_rows(hv, hq, pos, Hq, scale, gate=hg)
         reps += 1
         dt = time.perf_counter() - t0
         if dt > 10.0:
             break
+    ma, rl = I.errors(out_gpu.cpu().numpy(), ref)
+    model, ncpu = host_cpu()
     bytes_ = 2 * n_ctx * O.row_bytes(O.KV_Q8_0, Hkv, D)
-    return {"value": bytes_ * reps / dt / 1e9, "unit": "GB/s", "cores": int(O.lib().orc_num_threads()), "kind": "port",
-            "sample": f"{reps} full decode steps (1 row, ctx {n_ctx}, q8_0) of the C oracle with OpenMP, {dt:.1f} s"}, out, (q, gate, c)
+    return {"value": round(bytes_ * reps / dt / 1e9, 2), "unit": "GB/s", "cores": int(O.lib().orc_num_threads()), "kind": "port",
+            "sample": f"{reps} full decode steps (1 row, ctx {n_ctx}, q8_0, the pool and page table of the GPU's last timed step) of "
+                      f"the C oracle with OpenMP, {dt:.1f} s",
+            "cpu_model": model, "nproc": ncpu,
+            "gpu_output_check": {"max_abs": float(f"{ma:.3e}"), "rel_l2": float(f"{rl:.3e}"), "tol": [I.MAX_ABS_TOL, I.REL_L2_TOL],
+                                 "ok": bool(ma <= I.MAX_ABS_TOL and rl <= I.REL_L2_TOL)}}
+
+
+def cpu_prefill(torch, kv, ppseq, q, gate, out_gpu, p0, T, Hq, Hkv, D, psh, scale, every=32):
+    """the prefill half of the metric on the host: the oracle on every 32nd row of the chunk (128 of 4096 rows, each over
+    its 28673..32768 visible keys), timed once; the same rows check the GPU's output"""
+    import numpy as np
+    import _inputs as I
+    import _oracle as O
+    hv = host_view(torch, kv, ppseq, 0, Hkv, D, psh, O.KV_Q8_0)
+    rows = np.arange(every - 1, T, every)
+    hq, hg = q.cpu().numpy()[rows], gate.cpu().numpy()[rows]
+    pos = (p0 + rows).astype(np.int32)
+    t0 = time.perf_counter()
+    ref = O.attn_rows(hv, hq, pos, Hq, scale, gate=hg)
+    dt = time.perf_counter() - t0
+    flop = float(sum(4.0 * D * Hq * (int(p) + 1) for p in pos))
+    ma, rl = I.errors(out_gpu.cpu().numpy()[rows], ref)
+    model, ncpu = host_cpu()
+    return {"value": round(flop / dt / 1e12, 4), "unit": "TFLOP/s", "cores": int(O.lib().orc_num_threads()), "kind": "port",
+            "sample": f"{len(rows)} of {T} rows (every {every}th) of configs[4] on the C oracle with OpenMP, {dt:.1f} s; the full "
+                      f"chunk would take about {dt * T / len(rows):.0f} s",
+            "cpu_model": model, "nproc": ncpu,
+            "gpu_output_check": {"max_abs": float(f"{ma:.3e}"), "rel_l2": float(f"{rl:.3e}"), "tol": [I.MAX_ABS_TOL, I.REL_L2_TOL],
+                                 "ok": bool(ma <= I.MAX_ABS_TOL and rl <= I.REL_L2_TOL)}}
 
 
 def main():
@@ -335,15 +414,18 @@ def main():
     def step(i):
         return lambda: p1a.attn_decode(q, slots[i % n_pools], out, 1, n_ctx - 1, Hq, scale, gate=gate)
 
+    def kstep(i):   # the split-K kernel alone (a benchmarks-only entry point of the library: no merge, out untouched)
+        return lambda: p1a.bench_decode_split_only(q, slots[i % n_pools], out, 1, n_ctx - 1, Hq, scale)
+
     K, W = args.steps, args.warmup
     torch.cuda.synchronize()
-    sec = time_graph(torch, stream, [step(i) for i in range(K)], W)
+    # the dominant kernel alone first, so that the LAST thing to write `out` is the timed headline graph
+    sec_kernel = time_graph(torch, stream, [kstep(i) for i in range(K)], W)
+    sec_kernel_same = None if args.rotating_only else time_graph(torch, stream, [kstep(0) for _ in range(K)], W)
     sec_same = None if args.rotating_only else time_graph(torch, stream, [step(0) for _ in range(K)], W)
-    # the dominant kernel alone (the split-K kernel; the merge kernel is switched off for this graph only)
-    p1a.bench_skip_merge(True)
-    sec_kernel = time_graph(torch, stream, [step(i) for i in range(K)], W)
-    sec_kernel_same = None if args.rotating_only else time_graph(torch, stream, [step(0) for _ in range(K)], W)
-    p1a.bench_skip_merge(False)
+    out.fill_(float("nan"))
+    sec, samples = time_graph(torch, stream, [step(i) for i in range(K)], W, all_samples=True)
+    out_timed = out.clone()                                                # the result of step K - 1 of the last timed replay
     gbs = step_bytes / sec / 1e9
     kgbs = step_bytes / sec_kernel / 1e9
     traffic = None
@@ -356,12 +438,16 @@ def main():
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "q8_0 KV -> f16 MFMA, f32 accumulate", "data": "synthetic",
         "config": {"workload": "configs[1]: decode 24/4 heads, head_dim 256, ctx 32768, q8_0, 256-token pages, random page table",
-                   "kv_bytes_per_step": step_bytes, "pools_rotated": n_pools, "launch": "hipGraph of K steps"},
+                   "kv_bytes_per_step": step_bytes, "pools_rotated": n_pools,
+                   "launch": f"hipGraph of K steps, replayed {REPLAYS} times, median replay"},
+        "replay_ms_per_step": [round(x * 1e3, 5) for x in samples],
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": "dec_mfma_k<q8_0, 256, 1, 8>",
                      "kernel_us": round(sec_kernel * 1e6, 2),
                      "note": "achieved = algorithmic KV bytes of one launch (2 * ctx * 1088 B) / average duration of the "
-                             "split-K kernel, event-timed on its stream over a graph of K launches on rotating pools"},
+                             "split-K kernel, event-timed on its stream over a graph of K launches on rotating pools (median of "
+                             f"{REPLAYS} replays); traffic = HBM bytes per launch read from the committed rocprofv3 counter summary "
+                             "(profiles/decode_q8_0_32k_traffic.json), not measured in this run"},
         "extra": {"same_pool_GBs": sec_same and round(step_bytes / sec_same / 1e9, 1), "same_pool_us": sec_same and round(sec_same * 1e6, 2),
                   "kernel_same_pool_us": sec_kernel_same and round(sec_kernel_same * 1e6, 2),
                   "kernel_same_pool_GBs": sec_kernel_same and round(step_bytes / sec_kernel_same / 1e9, 1),
@@ -381,11 +467,16 @@ def main():
             torch.mul(src, 1.0, out=dst)                                   # reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del src, dst
-    if not args.no_extra:
-        res["extra"].update(extras(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     if not args.no_cpu:
-        cb, ref, (hq, hgate, hc) = cpu_baseline(Hq, Hkv, D, n_ctx, seed=7)
-        res["cpu_baseline"] = cb
+        res["cpu_baseline"] = cpu_baseline(torch, kv, ppseq, (K - 1) % n_pools, q, gate, out_timed, Hq, Hkv, D, psh, n_ctx, scale)
+    del kv, slots
+    if not args.no_extra:
+        top = {}
+        res["extra"].update(extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, not args.no_cpu))
+        if "roofline_prefill" in top:
+            res["roofline_prefill"] = top["roofline_prefill"]
+        if "cpu_prefill" in top:
+            res["cpu_baseline"]["prefill"] = top["cpu_prefill"]
     print(json.dumps(res))
 
 

@@ -144,6 +144,9 @@ inline bool attn_decode2(const float * q, const kv_cache & c, float * out, int T
 }
 inline int attn_dec2_nsplit(int Hkv) { return p1a_get_nsplit(Hkv); }
 inline void attn_dec2_set_nsplit(int n) { p1a_set_nsplit(n); }
+// src/fast/attn_dec2.cuh:21: re-read the environment switch baked into captured graphs (here P1A_DEC_SPLIT); true if it
+// changed, i.e. the caller's graphs must be dropped (src/tp_model.cu:3229)
+inline bool attn_dec2_reload_env() { return p1a_reload_env() != 0; }
 
 // src/fast/attn.cuh:46-53
 inline bool attn_prefill(const float * q, const kv_cache & c, float * out, int T, int p0, int Hq, float scale,

@@ -13,8 +13,10 @@
  *     untouched; a diagnostic goes to stderr and to p1a_last_error(). No exceptions, no host synchronisation.
  *   - Positions (`p0_dev`, `pos_rows`) and page tables (`pt`, `rtab`) are read ON THE DEVICE when the kernels run,
  *     so a captured hipGraph replays correctly at any depth.
- *   - Split-K scratch is owned by the library per (device, stream) and is allocated on the first call; call
- *     p1a_warmup() (or one eager call at the largest row count) before hipGraph capture so the pointer never changes.
+ *   - Split-K scratch is owned by the library per (device, stream). It is allocated on the first decode call (or by
+ *     p1a_warmup) at the footprint of P1A_MAX_ROWS rows of that call's head shape and is never freed or moved while the
+ *     library is loaded (p1a_release() frees everything), so a captured hipGraph stays valid whatever is called later
+ *     on its stream. Nothing is allocated during stream capture: warm up (or make one eager call) first.
  */
 #ifndef P1A_ATTN_H
 #define P1A_ATTN_H
@@ -172,31 +174,45 @@ size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D);
  * context (the last chunk of a prompt, a short turn of a long chat) would occupy T/128 * Hq workgroups, each walking every
  * key; its keys are then dealt to several workgroups per (token block, q head) and the partials merged (the nsplit of
  * attn_fold, src/fast/attn_fold.cuh:19-26, chosen by the library). The count depends on (T, p0, Hq) and the device's CU
- * count only, never on the scratch passed; partials that do not fit the caller's scratch live in the library's own
- * per-stream buffers (those of p1a_attn_decode; during stream capture they cannot grow and the call takes one split). */
+ * count only, never on the scratch passed or on the state of the stream; partials that do not fit the caller's scratch
+ * live in buffers the library keeps per (device, stream) for this purpose (never freed before p1a_release). They cannot
+ * be allocated during stream capture: such a call is refused with P1A_E_SCRATCH unless p1a_warmup_prefill (or an eager
+ * call of the shape) came first. */
 int p1a_attn_prefill_key_splits(int T, int p0, int Hq);
+/* Allocate the library's key-split partial buffers of (current device, stream) for a prefill call of this shape (a no-op
+ * for shapes that take one split), so that the call can be captured. No counterpart in the reference, whose attn_fold
+ * takes all scratch from the caller (src/fast/attn_fold.cuh:25-26). */
+int p1a_warmup_prefill(int T, int p0, int Hq, int Hkv, int D, void *stream);
 
 /* Standalone sigmoid gate x[i] *= 1 / (1 + exp(-g[i])). Replaces k::sigmoid_mul, src/kernels.cu:85-93. */
 int p1a_sigmoid_mul(float *x, const float *g, size_t n, void *stream);
 
 /*
- * Allocate the split-K scratch of (current device, stream) for up to `rows` query rows of Hq heads of size D, so that
- * later calls on that stream never allocate (graph capture). Mirrors the warm-up call the reference asks for
- * (src/fast/attn.cuh:40-42).
+ * Allocate the split-K scratch of (current device, stream) for Hq heads of size D (always at the P1A_MAX_ROWS footprint:
+ * `rows` is only checked), so that later decode calls of that head shape on that stream never allocate (graph
+ * capture). Mirrors the warm-up call the reference asks for (src/fast/attn.cuh:40-42; the reference allocates at its
+ * ATTN_MAX_ROWS footprint on first use, src/fast/attn_dec2.cu:452-464,503-517).
  */
 int p1a_warmup(int rows, int Hq, int Hkv, int D, void *stream);
 /* split-stream count used for Hkv kv heads on the current device / override it (0 = default). Mirror
  * attn_dec2_nsplit / attn_dec2_set_nsplit, src/fast/attn_dec2.cuh:19-20. Never change it between graph captures. */
 int p1a_get_nsplit(int Hkv);
 void p1a_set_nsplit(int n);
-/* Benchmarks only (no counterpart in the reference, whose benches time both kernels together): when on,
- * p1a_attn_decode stops after the split-K kernel and leaves `out` untouched, so that kernel can be event-timed alone. */
-void p1a_bench_skip_merge(int on);
+/* Re-read the environment switch that is baked into captured graphs (P1A_DEC_SPLIT, the split-stream count); returns 1
+ * when it changed since it was last read (the caller must then drop its captured graphs), else 0.
+ * Replaces attn_dec2_reload_env, src/fast/attn_dec2.cuh:21 (called from src/tp_model.cu:3229). */
+int p1a_reload_env(void);
+/* Benchmarks only (no counterpart in the reference, whose benches time both kernels together): p1a_attn_decode without
+ * its merge kernel - the split-K kernel runs and leaves its partials in the library's scratch, `out` is untouched - so
+ * that kernel can be event-timed alone. The flag is an argument of this call: no process-wide state. */
+int p1a_bench_decode_split_only(const float *q, const p1a_kv *c, float *out, int T, int p0, const int32_t *p0_dev,
+                                const int32_t *pos_rows, int rows_per_seq, int Hq, float scale, void *stream);
 /* Benchmarks only (no counterpart in the reference): a plain read of `bytes` bytes of device memory (16 bytes per lane,
  * one contiguous span per workgroup, nothing computed) - the time the memory system needs for a launch of that size,
  * to set a decode launch of the same number of KV bytes against. bytes is rounded down to a multiple of 16. */
 int p1a_bench_stream_read(const void *src, size_t bytes, void *stream);
-/* free every scratch buffer of the current process (after synchronising the devices that own them) */
+/* free every scratch buffer of the current process (after synchronising the devices that own them); graphs captured
+ * before this call must not be replayed after it */
 void p1a_release(void);
 
 const char *p1a_last_error(void);

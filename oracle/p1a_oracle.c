@@ -197,9 +197,60 @@ void orc_rmsnorm_heads(float *x, size_t nheads, int D, float eps) {
  * codes can be compared bit for bit): the sum of squares is formed per group of 4 consecutive dims, left to right,
  * and the groups are added in a balanced binary tree over 64 slots (empty slots are 0); the scale is 1 / sqrtf(...)
  * with IEEE division and square root (the reference uses the approximate rsqrtf, a difference of an ulp); the
- * rotation angle is pos * (float) pow(base, -2j/n_rot) in fp32 and its cosine / sine are the double-precision ones
- * rounded to fp32; products and sums are rounded separately (no fused multiply-add).
+ * rotation angle is pos * (float) base^(-2j/n_rot) in fp32 and its cosine / sine are rounded to fp32 (the reference
+ * calls CUDA's powf / cosf / sinf, fused.cu:551-553, whose last bits no other machine reproduces); products and sums
+ * are rounded separately (no fused multiply-add).
+ * Power, cosine and sine are spelled out below in IEEE double operations in a fixed order - NOT taken from libm - so
+ * that the result bits do not depend on the math library: ln by the atanh series on the frexp mantissa, e^x by
+ * Cody-Waite reduction with a degree-13 Taylor polynomial, sin / cos by reduction against pi/2 held in four 24-bit
+ * pieces and the fdlibm kernel polynomials. tests/test_oracle_prep.py pins them against numpy's float64 functions.
  */
+static double prep_log(double x) {
+    const double LN2_HI = 6.93147180369123816490e-01, LN2_LO = 1.90821492927058770002e-10;
+    int e = 0;
+    double m = frexp(x, &e);
+    if (m < 7.07106781186547524401e-01) { m = m * 2.0; e -= 1; }
+    const double s = (m - 1.0) / (m + 1.0), z = s * s;
+    double p = 1.0 / 25.0;
+    for (int k = 23; k >= 1; k -= 2) p = p * z + 1.0 / (double) k;
+    const double lm = (2.0 * s) * p;
+    return (double) e * LN2_HI + ((double) e * LN2_LO + lm);
+}
+static double prep_exp(double x) {
+    const double LOG2E = 1.44269504088896338700e+00, LN2_HI = 6.93147180369123816490e-01, LN2_LO = 1.90821492927058770002e-10;
+    static const double inv_fact[14] = {1.0, 1.0, 0.5, 1.0 / 6.0, 1.0 / 24.0, 1.0 / 120.0, 1.0 / 720.0, 1.0 / 5040.0, 1.0 / 40320.0,
+                                        1.0 / 362880.0, 1.0 / 3628800.0, 1.0 / 39916800.0, 1.0 / 479001600.0, 1.0 / 6227020800.0};
+    const double k = rint(x * LOG2E);
+    const double r = (x - k * LN2_HI) - k * LN2_LO;
+    double p = inv_fact[13];
+    for (int i = 12; i >= 0; --i) p = p * r + inv_fact[i];
+    return ldexp(p, (int) k);
+}
+static void prep_sincos(double t, float *c, float *s) {
+    static const double pio2[4] = {1.57079625129699707031e+00, 7.54978941586159635335e-08, 5.39030252995776476554e-15, 3.28200341580791294123e-22};
+    static const double S[6] = {-1.66666666666666324348e-01, 8.33333333332248946124e-03, -1.98412698298579493134e-04,
+                                2.75573137070700676789e-06, -2.50507602534068634195e-08, 1.58969099521155010221e-10};
+    static const double C[6] = {4.16666666666666019037e-02, -1.38888888888741095749e-03, 2.48015872894767294178e-05,
+                                -2.75573143513906633035e-07, 2.08757232129817482790e-09, -1.13596475577881948265e-11};
+    const double n = rint(t * 6.36619772367581382433e-01);
+    double r = t;
+    for (int i = 0; i < 4; ++i) r = r - n * pio2[i];
+    const double z = r * r;
+    double ps = S[4] + z * S[5], pc = C[4] + z * C[5];
+    for (int i = 3; i >= 0; --i) { ps = S[i] + z * ps; pc = C[i] + z * pc; }
+    const double sn = r + (z * r) * ps;
+    const double cs = 1.0 - (0.5 * z - (z * z) * pc);
+    switch ((int) ((long long) n & 3)) {
+        case 0: *c = (float) cs; *s = (float) sn; break;
+        case 1: *c = (float) -sn; *s = (float) cs; break;
+        case 2: *c = (float) -cs; *s = (float) -sn; break;
+        default: *c = (float) sn; *s = (float) -cs; break;
+    }
+}
+/* exported for the tests that pin the three recipes */
+double orc_prep_inv_freq(float freq_base, int j, int n_rot) { return prep_exp(((-2.0 * (double) j) / (double) n_rot) * prep_log((double) freq_base)); }
+void orc_prep_sincos(float theta, float *c, float *s) { prep_sincos((double) theta, c, s); }
+
 /* interleaved M-RoPE (src/fast/mrope.cuh:1-8, 25-33): rotary pair j takes the position of one of three streams by its
  * sector = j % sect: sector % 3 == 1 and < 3 s1 -> h; sector % 3 == 2 and < 3 s2 -> w; sector % 3 == 0 and < 3 s0 -> t;
  * anything else -> the 4th stream, which is 0. mr == NULL: every pair takes pos. */
@@ -236,10 +287,12 @@ static void prep_norm_rope(const float *src, const float *w, int D, int n_rot, f
         dst[i] = o;
     }
     const int half = n_rot / 2;
+    const double ln_base = prep_log((double) freq_base);
     for (int j = 0; j < half; ++j) {
-        const float inv = (float) pow((double) freq_base, -2.0 * (double) j / (double) n_rot);
+        const float inv = (float) prep_exp(((-2.0 * (double) j) / (double) n_rot) * ln_base);
         const float theta = (float) mrope_pick(mr, t, j, pos) * inv;
-        const float c = (float) cos((double) theta), sn = (float) sin((double) theta);
+        float c, sn;
+        prep_sincos((double) theta, &c, &sn);
         const float x0 = dst[j], x1 = dst[j + half];
         const float a0 = x0 * c, a1 = x1 * sn, b0 = x0 * sn, b1 = x1 * c;
         dst[j] = a0 - a1;

@@ -17,6 +17,9 @@
  *   orc_attn_prep                              : numpy float64 restatement of norm * weight and the NEOX rotation (to a few
  *       fp32 ulps); closed forms (position 0 rotates nothing, the rotation keeps pair norms, q . k after rope depends on
  *       the position difference only, a constant head norms to w); KV rows == orc_kv_append_rows of the normed, roped k.
+ *       Its power / cosine / sine recipes (IEEE double operations in a fixed order, no libm: orc_prep_inv_freq,
+ *       orc_prep_sincos) against numpy's float64 pow / cos / sin rounded to fp32: equal but for rare last-bit roundings
+ *       (the double result sits within 2^-50 of a rounding boundary), over all rotary pairs and angles up to 2^29.
  *   orc_attn_prep_mrope                        : t = h = w = p is bitwise plain NEOX at p (src/fast/mrope.cuh:6-7); the
  *       stream of every rotary pair from a table written out by hand from the rule's words for sections [11, 11, 10, 0]
  *       and [2, 1, 1, 0]; moving one stream changes exactly the pairs of that stream.
@@ -91,6 +94,10 @@ typedef struct orc_mrope {
 int orc_attn_prep_mrope(const float *qg, const float *k, const float *v, const float *q_norm, const float *k_norm,
                         const int32_t *pos, float *q, float *gate, const orc_kv *c, int p0, int T, int Hq, int Hkv, int D,
                         int n_rot, float freq_base, float eps, int ldq, int ldk, int ldv, const orc_mrope *mr);
+/* the rotary recipes of orc_attn_prep, exported for the tests that pin them: base^(-2j/n_rot) in double, and the fp32
+ * cosine / sine of an fp32 angle */
+double orc_prep_inv_freq(float freq_base, int j, int n_rot);
+void orc_prep_sincos(float theta, float *c, float *s);
 /* a16 activation quantize (src/fast/a16q.cuh:21-45 = src/fast/matvec_a16.cu:29-100): y [T][n] f32, n % 32 == 0 ->
  * qbuf: T * n/32 * 16 half2 of scaled values (slot order of the engine), then T * n/32 half2 (amax, sum). */
 void orc_a16_quant(const float *y, int T, int n, uint16_t *qbuf);

@@ -8,7 +8,7 @@ KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
     "p1a_kv_row_bytes", "p1a_kv_append", "p1a_kv_fill_random", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
-    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_bench_skip_merge", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
+    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_reload_env", "p1a_warmup_prefill", "p1a_bench_decode_split_only", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
     "p1a_version",
     # include/p1a_pool.h
     "p1a_pool_create", "p1a_pool_destroy", "p1a_pool_n_pages", "p1a_pool_free_pages", "p1a_pool_max_pages", "p1a_pool_page_bytes",
@@ -91,8 +91,12 @@ def lib():
     L.p1a_get_nsplit.argtypes = [i32]
     L.p1a_set_nsplit.restype = None
     L.p1a_set_nsplit.argtypes = [i32]
-    L.p1a_bench_skip_merge.restype = None
-    L.p1a_bench_skip_merge.argtypes = [i32]
+    L.p1a_reload_env.restype = i32
+    L.p1a_reload_env.argtypes = []
+    L.p1a_warmup_prefill.restype = i32
+    L.p1a_warmup_prefill.argtypes = [i32, i32, i32, i32, i32, vp]
+    L.p1a_bench_decode_split_only.restype = i32
+    L.p1a_bench_decode_split_only.argtypes = [vp, kvp, vp, i32, i32, vp, vp, i32, i32, f32, vp]
     L.p1a_bench_stream_read.restype = i32
     L.p1a_bench_stream_read.argtypes = [vp, sz, vp]
     L.p1a_release.restype = None
@@ -318,8 +322,18 @@ def set_nsplit(n):
     lib().p1a_set_nsplit(n)
 
 
-def bench_skip_merge(on):
-    lib().p1a_bench_skip_merge(1 if on else 0)
+def reload_env():
+    """src/fast/attn_dec2.cuh:21: True when the split-count environment switch changed (captured graphs must be dropped)."""
+    return bool(lib().p1a_reload_env())
+
+
+def warmup_prefill(T, p0, Hq, Hkv, D):
+    _check(lib().p1a_warmup_prefill(T, p0, Hq, Hkv, D, _stream()), "warmup_prefill")
+
+
+def bench_decode_split_only(q, c, out, T, p0, Hq, scale, pos=None, rows_per_seq=0):
+    """Benchmarks only: the split-K kernel of attn_decode / attn_decode_rows without the merge (out untouched)."""
+    _check(lib().p1a_bench_decode_split_only(_ptr(q), ctypes.byref(c.struct()), _ptr(out), T, p0, None, _ptr(pos), rows_per_seq, Hq, scale, _stream()), "bench_decode_split_only")
 
 
 def bench_stream_read(t):

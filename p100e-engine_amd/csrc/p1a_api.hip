@@ -22,15 +22,24 @@ void set_error(const char * fmt, ...) {
 
 namespace {
 
-// Split partials per (device, stream): calls on different streams of one device may overlap; a stream keeps its
-// buffer (captured graphs hold the pointer), which only ever grows, and only outside capture.
-struct scratch { int dev = -1; hipStream_t s = nullptr; float * o = nullptr; float * ml = nullptr; size_t cap_o = 0, cap_ml = 0; };
+// Split partials per (device, stream): calls on different streams of one device may overlap. A captured graph holds the
+// pointers it was recorded with, so a buffer is NEVER freed while the library lives: the decode buffers are allocated on
+// the first call at the footprint of P1A_MAX_ROWS rows of that call's head shape (every KV type and row grouping), and
+// in the rare case that a later call needs more (another head shape, a larger split count) the new buffer replaces the
+// old one only for later calls - the old one stays allocated (g_retired) until p1a_release(). Nothing is allocated
+// while the stream is being captured. The partials of a key-split prefill have a pair of their own.
+struct bufpair { float * o = nullptr; float * ml = nullptr; size_t cap_o = 0, cap_ml = 0; };
+struct scratch { int dev = -1; hipStream_t s = nullptr; bufpair dec, pf; };
 constexpr int MAX_SCR = 64;
+constexpr int MAX_RETIRED = 1024;
 scratch g_scr[MAX_SCR];
 int g_nscr = 0;
+struct retired { int dev; void * p; };
+retired g_retired[MAX_RETIRED];
+int g_nretired = 0;
 std::mutex g_mu;
 int g_nsplit_override = 0;
-bool g_skip_merge = false;
+int g_env_split = -1;   // P1A_DEC_SPLIT as last read (-1 = not read yet)
 int g_cus[16] = {0};
 
 }   // namespace
@@ -45,7 +54,10 @@ int cu_count() {
 
 namespace {
 
-scratch * scratch_for(hipStream_t s, size_t need_o, size_t need_ml, bool quiet = false) {
+enum which_buf { BUF_DECODE, BUF_PREFILL };
+
+// the buffer pair `w` of (current device, s) with at least these capacities, or nullptr (error set unless quiet)
+bufpair * scratch_for(hipStream_t s, which_buf w, size_t need_o, size_t need_ml, bool quiet = false) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lk(g_mu);
@@ -56,12 +68,16 @@ scratch * scratch_for(hipStream_t s, size_t need_o, size_t need_ml, bool quiet =
         e = &g_scr[g_nscr++];
         e->dev = dev; e->s = s;
     }
-    if (need_o > e->cap_o || need_ml > e->cap_ml) {
+    bufpair & b = w == BUF_DECODE ? e->dec : e->pf;
+    if (need_o > b.cap_o || need_ml > b.cap_ml) {
         hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
         if (s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone) {
-            if (!quiet) set_error("split scratch would have to grow during stream capture: call p1a_warmup first");
+            if (!quiet) set_error("split scratch would have to be allocated during stream capture: call p1a_warmup%s first", w == BUF_PREFILL ? "_prefill" : "");
             return nullptr;
         }
+        if (b.o && g_nretired + 2 > MAX_RETIRED) { if (!quiet) set_error("split scratch replaced too often"); return nullptr; }
+        if (need_o < b.cap_o) need_o = b.cap_o;
+        if (need_ml < b.cap_ml) need_ml = b.cap_ml;
         float * no = nullptr, * nm = nullptr;
         if (hipMalloc(&no, need_o) != hipSuccess || hipMalloc(&nm, need_ml) != hipSuccess) {
             (void) hipGetLastError();
@@ -69,10 +85,11 @@ scratch * scratch_for(hipStream_t s, size_t need_o, size_t need_ml, bool quiet =
             if (!quiet) set_error("split scratch allocation failed (%zu bytes)", need_o + need_ml);
             return nullptr;
         }
-        if (e->o) { (void) hipStreamSynchronize(s); (void) hipFree(e->o); (void) hipFree(e->ml); }
-        e->o = no; e->ml = nm; e->cap_o = need_o; e->cap_ml = need_ml;
+        // the replaced buffers stay allocated: a graph captured earlier on this stream may still write and read them
+        if (b.o) { g_retired[g_nretired++] = retired{dev, b.o}; g_retired[g_nretired++] = retired{dev, b.ml}; }
+        b.o = no; b.ml = nm; b.cap_o = need_o; b.cap_ml = need_ml;
     }
-    return e;
+    return &b;
 }
 
 bool kv_ok(const p1a_kv * c, const char * who) {
@@ -84,15 +101,80 @@ bool kv_ok(const p1a_kv * c, const char * who) {
 }
 
 // requested split-stream count: the setter, then the environment, else 0 = the plan's default for the device
+int read_env_split() {
+    const char * e = getenv("P1A_DEC_SPLIT");
+    const int v = e && *e ? atoi(e) : 0;
+    return v > 0 ? v : 0;
+}
 int nsplit_req() {
-    static const int env = getenv("P1A_DEC_SPLIT") ? atoi(getenv("P1A_DEC_SPLIT")) : 0;
-    return g_nsplit_override > 0 ? g_nsplit_override : (env > 0 ? env : 0);
+    if (g_env_split < 0) g_env_split = read_env_split();
+    return g_nsplit_override > 0 ? g_nsplit_override : g_env_split;
+}
+
+// the decode split buffers of a head shape: P1A_MAX_ROWS rows, the largest need over the KV types and row groupings
+void decode_footprint(int Hq, int Hkv, int D, size_t & need_o, size_t & need_ml) {
+    p1a_kv c;
+    memset(&c, 0, sizeof c);
+    c.Hkv = Hkv; c.D = D; c.k = c.v = (void *) 16;
+    need_o = need_ml = 0;
+    const uint32_t types[3] = {P1A_KV_F16, P1A_KV_Q8_0, P1A_KV_Q4_0};
+    for (uint32_t ty : types)
+        for (int rg = 1; rg <= 4; ++rg) {
+            size_t o, m;
+            c.type = ty;
+            decode_scratch_need(c, Hq, P1A_MAX_ROWS, rg, nsplit_req(), cu_count(), o, m);
+            if (o > need_o) need_o = o;
+            if (m > need_ml) need_ml = m;
+        }
+}
+
+// ext / ext_bytes: split scratch brought by the caller of this function (the allocation-free entry point); nullptr = the
+// library's own per-stream buffers
+int decode_call(const float * q, const p1a_kv * c, float * out, const float * gate, void * qbuf, int T, int p0,
+                const int32_t * p0_dev, const int32_t * pos_rows, int rows_per_seq, int Hq, float scale, bool split_only,
+                hipStream_t s, void * ext = nullptr, size_t ext_bytes = 0) {
+    if (!kv_ok(c, "p1a_attn_decode")) return P1A_E_ARG;
+    if (qbuf && (((uintptr_t) qbuf & 15) || (Hq * c->D) % 32)) { set_error("p1a_attn_decode: qbuf must be 16-byte aligned and Hq*D %% 32 == 0"); return P1A_E_SHAPE; }
+    if (!q || !out) { set_error("p1a_attn_decode: null q/out"); return P1A_E_ARG; }
+    if (T < 1 || T > P1A_MAX_ROWS || Hq < c->Hkv || Hq % c->Hkv) {
+        set_error("p1a_attn_decode: unsupported shape (D=%d Hq=%d Hkv=%d T=%d)", c->D, Hq, c->Hkv, T);
+        return P1A_E_SHAPE;
+    }
+    if ((((uintptr_t) q | (uintptr_t) out | (uintptr_t) gate) & 15)) { set_error("p1a_attn_decode: q/out/gate must be 16-byte aligned"); return P1A_E_SHAPE; }
+    if (!pos_rows && !p0_dev && p0 < 0) { set_error("p1a_attn_decode: negative p0"); return P1A_E_ARG; }
+    decode_args a;
+    a.q = q; a.out = out; a.gate = gate; a.T = T; a.p0 = p0; a.p0_dev = p0_dev; a.pos_rows = pos_rows;
+    a.Hq = Hq; a.scale = scale;
+    a.rows_per_group = decode_rows_per_group(*c, Hq, pos_rows ? (rows_per_seq < 1 ? 1 : rows_per_seq) : T);
+    // a sequence's rows must split into whole groups, or a group would mix two sequences
+    while (pos_rows && rows_per_seq > 1 && rows_per_seq % a.rows_per_group) --a.rows_per_group;
+    a.nsplit = nsplit_req();
+    a.cus = cu_count();
+    a.skip_merge = split_only;
+    a.qbuf = qbuf;
+    size_t need_o, need_ml;
+    if (ext) {
+        decode_scratch_need(*c, Hq, T, a.rows_per_group, a.nsplit, a.cus, need_o, need_ml);
+        need_o = (need_o + 255) & ~(size_t) 255;
+        if (need_o + need_ml > ext_bytes) {
+            set_error("p1a_attn_decode_noalloc: this call needs %zu bytes of split scratch, the static buffer holds %zu", need_o + need_ml, ext_bytes);
+            return P1A_E_SCRATCH;
+        }
+        a.part_o = reinterpret_cast<float *>(ext);
+        a.part_ml = reinterpret_cast<float *>(reinterpret_cast<char *>(ext) + need_o);
+        return launch_decode(*c, a, s);
+    }
+    decode_footprint(Hq, c->Hkv, c->D, need_o, need_ml);
+    bufpair * sc = scratch_for(s, BUF_DECODE, need_o, need_ml);
+    if (!sc) return P1A_E_SCRATCH;
+    a.part_o = sc->o; a.part_ml = sc->ml;
+    return launch_decode(*c, a, s);
 }
 
 }   // namespace
 
 bool split_scratch(hipStream_t s, size_t bytes_o, size_t bytes_ml, float *& o, float *& ml) {
-    scratch * e = scratch_for(s, bytes_o, bytes_ml, true);
+    bufpair * e = scratch_for(s, BUF_PREFILL, bytes_o, bytes_ml);
     if (!e) return false;
     o = e->o; ml = e->ml;
     return true;
@@ -151,6 +233,7 @@ int p1a_attn_prep_mrope(const float * qg, const float * k, const float * v, cons
         set_error("p1a_attn_prep: unsupported shape (D=%d n_rot=%d T=%d): D <= 256, n_rot %% 8 == 0, n_rot <= D", D, n_rot, T);
         return P1A_E_SHAPE;
     }
+    if (!(freq_base > 0.0f) || !(freq_base < 3.0e38f)) { set_error("p1a_attn_prep: freq_base must be a positive finite number"); return P1A_E_ARG; }
     if (!ldq) ldq = Hq * 2 * D;
     if (!ldk) ldk = Hkv * D;
     if (!ldv) ldv = Hkv * D;
@@ -187,51 +270,27 @@ int p1a_attn_decode(const float * q, const p1a_kv * c, float * out, const float 
 int p1a_attn_decode_a16(const float * q, const p1a_kv * c, float * out, const float * gate, void * qbuf, int T, int p0,
                         const int32_t * p0_dev, const int32_t * pos_rows, int rows_per_seq, int Hq, float scale,
                         void * stream) {
-    if (!kv_ok(c, "p1a_attn_decode")) return P1A_E_ARG;
-    if (qbuf && (((uintptr_t) qbuf & 15) || (Hq * c->D) % 32)) { set_error("p1a_attn_decode: qbuf must be 16-byte aligned and Hq*D %% 32 == 0"); return P1A_E_SHAPE; }
-    if (!q || !out) { set_error("p1a_attn_decode: null q/out"); return P1A_E_ARG; }
-    if (T < 1 || T > P1A_MAX_ROWS || Hq < c->Hkv || Hq % c->Hkv) {
-        set_error("p1a_attn_decode: unsupported shape (D=%d Hq=%d Hkv=%d T=%d)", c->D, Hq, c->Hkv, T);
-        return P1A_E_SHAPE;
-    }
-    if ((((uintptr_t) q | (uintptr_t) out | (uintptr_t) gate) & 15)) { set_error("p1a_attn_decode: q/out/gate must be 16-byte aligned"); return P1A_E_SHAPE; }
-    if (!pos_rows && !p0_dev && p0 < 0) { set_error("p1a_attn_decode: negative p0"); return P1A_E_ARG; }
-    hipStream_t s = (hipStream_t) stream;
-    decode_args a;
-    a.q = q; a.out = out; a.gate = gate; a.T = T; a.p0 = p0; a.p0_dev = p0_dev; a.pos_rows = pos_rows;
-    a.Hq = Hq; a.scale = scale;
-    a.rows_per_group = decode_rows_per_group(*c, Hq, pos_rows ? (rows_per_seq < 1 ? 1 : rows_per_seq) : T);
-    // a sequence's rows must split into whole groups, or a group would mix two sequences
-    while (pos_rows && rows_per_seq > 1 && rows_per_seq % a.rows_per_group) --a.rows_per_group;
-    a.nsplit = nsplit_req();
-    a.cus = cu_count();
-    a.skip_merge = g_skip_merge;
-    a.qbuf = qbuf;
-    size_t need_o, need_ml;
-    decode_scratch_need(*c, Hq, T < 8 ? 8 : T, a.rows_per_group, a.nsplit, a.cus, need_o, need_ml);
-    scratch * sc = scratch_for(s, need_o, need_ml);
-    if (!sc) return P1A_E_SCRATCH;
-    a.part_o = sc->o; a.part_ml = sc->ml;
-    return launch_decode(*c, a, s);
+    return decode_call(q, c, out, gate, qbuf, T, p0, p0_dev, pos_rows, rows_per_seq, Hq, scale, false, (hipStream_t) stream);
+}
+
+int p1a_bench_decode_split_only(const float * q, const p1a_kv * c, float * out, int T, int p0, const int32_t * p0_dev,
+                                const int32_t * pos_rows, int rows_per_seq, int Hq, float scale, void * stream) {
+    return decode_call(q, c, out, nullptr, nullptr, T, p0, p0_dev, pos_rows, rows_per_seq, Hq, scale, true, (hipStream_t) stream);
 }
 
 int p1a_warmup(int rows, int Hq, int Hkv, int D, void * stream) {
     if (rows < 1 || rows > P1A_MAX_ROWS || Hq < 1 || Hkv < 1 || Hq % Hkv || D < 32) { set_error("p1a_warmup: bad shape"); return P1A_E_ARG; }
-    // the largest footprint over the kernels and row groupings a (Hq, Hkv, D) cache can take
-    p1a_kv c;
-    memset(&c, 0, sizeof c);
-    c.Hkv = Hkv; c.D = D; c.k = c.v = (void *) 16;
-    size_t need_o = 0, need_ml = 0;
-    const uint32_t types[3] = {P1A_KV_F16, P1A_KV_Q8_0, P1A_KV_Q4_0};
-    for (uint32_t ty : types)
-        for (int rg = 1; rg <= 4; ++rg) {
-            size_t o, m;
-            c.type = ty;
-            decode_scratch_need(c, Hq, rows < 8 ? 8 : rows, rg, nsplit_req(), cu_count(), o, m);
-            if (o > need_o) need_o = o;
-            if (m > need_ml) need_ml = m;
-        }
-    return scratch_for((hipStream_t) stream, need_o, need_ml) ? P1A_OK : P1A_E_SCRATCH;
+    size_t need_o, need_ml;
+    decode_footprint(Hq, Hkv, D, need_o, need_ml);
+    return scratch_for((hipStream_t) stream, BUF_DECODE, need_o, need_ml) ? P1A_OK : P1A_E_SCRATCH;
+}
+
+int p1a_warmup_prefill(int T, int p0, int Hq, int Hkv, int D, void * stream) {
+    if (T < 1 || p0 < 0 || Hq < 1 || Hkv < 1 || Hq % Hkv || D < 32) { set_error("p1a_warmup_prefill: bad shape"); return P1A_E_ARG; }
+    size_t bo, bm;
+    prefill_part_need(T, p0, Hq, D, bo, bm);
+    if (!bo) return P1A_OK;
+    return scratch_for((hipStream_t) stream, BUF_PREFILL, bo, bm) ? P1A_OK : P1A_E_SCRATCH;
 }
 
 int p1a_attn_prefill(const float * q, const p1a_kv * c, float * out, const float * gate, int T, int p0, int Hq,
@@ -258,7 +317,12 @@ int p1a_get_nsplit(int Hkv) {
 
 void p1a_set_nsplit(int n) { g_nsplit_override = n > 0 ? n : 0; }
 
-void p1a_bench_skip_merge(int on) { g_skip_merge = on != 0; }
+int p1a_reload_env(void) {
+    const int v = read_env_split();
+    const bool changed = g_env_split >= 0 && v != g_env_split;
+    g_env_split = v;
+    return changed ? 1 : 0;
+}
 
 int p1a_bench_stream_read(const void * src, size_t bytes, void * stream) {
     if (!src || bytes < 16 || ((uintptr_t) src & 15)) { set_error("p1a_bench_stream_read: null, short or misaligned source"); return P1A_E_ARG; }
@@ -270,14 +334,18 @@ void p1a_release(void) {
     int cur = 0;
     (void) hipGetDevice(&cur);
     for (int i = 0; i < g_nscr; ++i) {
-        if (!g_scr[i].o) continue;
         (void) hipSetDevice(g_scr[i].dev);
         (void) hipDeviceSynchronize();
-        (void) hipFree(g_scr[i].o);
-        (void) hipFree(g_scr[i].ml);
+        for (bufpair * b : {&g_scr[i].dec, &g_scr[i].pf})
+            if (b->o) { (void) hipFree(b->o); (void) hipFree(b->ml); }
         g_scr[i] = scratch{};
     }
     g_nscr = 0;
+    for (int i = 0; i < g_nretired; ++i) {
+        (void) hipSetDevice(g_retired[i].dev);
+        (void) hipFree(g_retired[i].p);
+    }
+    g_nretired = 0;
     (void) hipSetDevice(cur);
 }
 

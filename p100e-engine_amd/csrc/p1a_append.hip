@@ -115,14 +115,86 @@ __global__ void __launch_bounds__(256) append_k(const float * __restrict__ k, co
 // (gate copy, norm, rope, store), Hq <= b < Hq + Hkv k heads (norm, rope, quantizing write), the rest v heads (write).
 // Operation order (the CPU oracle keeps the same one, so K codes compare bit for bit): the squares of a lane's 4 values
 // are added left to right, the 64 lane sums in a butterfly (a balanced binary tree); scale = 1 / sqrtf(ss / D + eps)
-// with IEEE division and square root; angle = pos * (float) pow(base, -2 j / n_rot) in fp32, cosine and sine in double
-// precision rounded to fp32; every product and sum rounded on its own.
+// with IEEE division and square root; angle = pos * (float) base^(-2 j / n_rot) in fp32, its cosine and sine rounded to
+// fp32 - power, cosine and sine through the fixed recipes below, not through a math library; every product and sum
+// rounded on its own.
+//
+// The elementary functions of the rotary angle are spelled out in IEEE double additions, multiplications, divisions and
+// round-to-integer, in a fixed order without contraction, so that any IEEE machine gets the same bits (two math
+// libraries differ in the last bit now and then, and a last bit moves a K code):
+//   ln x    : x = m 2^e with m in [sqrt(1/2), sqrt(2)); s = (m - 1) / (m + 1); ln m = 2 s (1 + s^2/3 + ... + s^24/25) (host)
+//   e^x     : k = rint(x log2 e); r = (x - k LN2_HI) - k LN2_LO; Taylor to r^13 in Horner form; scaled by 2^k
+//   sin, cos: n = rint(t 2/pi); r = t - n pi/2 with pi/2 in four 24-bit pieces (n a_i is exact for n < 2^29);
+//             the fdlibm kernel polynomials on |r| <= pi/4; quadrant n mod 4
+// each is within an ulp or two of double precision; the results are then rounded to fp32.
+__host__ __device__ inline double det_exp(double x) {
+    const double LOG2E = 1.44269504088896338700e+00, LN2_HI = 6.93147180369123816490e-01, LN2_LO = 1.90821492927058770002e-10;
+    const double k = __builtin_rint(x * LOG2E);
+    const double r = (x - k * LN2_HI) - k * LN2_LO;
+    double p = 1.0 / 6227020800.0;
+    p = p * r + 1.0 / 479001600.0;
+    p = p * r + 1.0 / 39916800.0;
+    p = p * r + 1.0 / 3628800.0;
+    p = p * r + 1.0 / 362880.0;
+    p = p * r + 1.0 / 40320.0;
+    p = p * r + 1.0 / 5040.0;
+    p = p * r + 1.0 / 720.0;
+    p = p * r + 1.0 / 120.0;
+    p = p * r + 1.0 / 24.0;
+    p = p * r + 1.0 / 6.0;
+    p = p * r + 0.5;
+    p = p * r + 1.0;
+    p = p * r + 1.0;
+    return __builtin_ldexp(p, (int) k);
+}
+__host__ __device__ inline void det_sincos(double t, float & c, float & s) {
+    const double TWO_OVER_PI = 6.36619772367581382433e-01;
+    const double A1 = 1.57079625129699707031e+00, A2 = 7.54978941586159635335e-08, A3 = 5.39030252995776476554e-15, A4 = 3.28200341580791294123e-22;
+    const double n = __builtin_rint(t * TWO_OVER_PI);
+    double r = t - n * A1;
+    r = r - n * A2;
+    r = r - n * A3;
+    r = r - n * A4;
+    const double z = r * r;
+    const double S1 = -1.66666666666666324348e-01, S2 = 8.33333333332248946124e-03, S3 = -1.98412698298579493134e-04;
+    const double S4 = 2.75573137070700676789e-06, S5 = -2.50507602534068634195e-08, S6 = 1.58969099521155010221e-10;
+    const double C1 = 4.16666666666666019037e-02, C2 = -1.38888888888741095749e-03, C3 = 2.48015872894767294178e-05;
+    const double C4 = -2.75573143513906633035e-07, C5 = 2.08757232129817482790e-09, C6 = -1.13596475577881948265e-11;
+    double ps = S5 + z * S6;
+    ps = S4 + z * ps;
+    ps = S3 + z * ps;
+    ps = S2 + z * ps;
+    ps = S1 + z * ps;
+    const double sn = r + (z * r) * ps;
+    double pc = C5 + z * C6;
+    pc = C4 + z * pc;
+    pc = C3 + z * pc;
+    pc = C2 + z * pc;
+    pc = C1 + z * pc;
+    const double cs = 1.0 - (0.5 * z - (z * z) * pc);
+    const int q = (int) ((long long) n & 3);
+    const double cc = q == 0 ? cs : q == 1 ? -sn : q == 2 ? -cs : sn;
+    const double ss = q == 0 ? sn : q == 1 ? cs : q == 2 ? -sn : -cs;
+    c = (float) cc;
+    s = (float) ss;
+}
+inline double det_log(double x) {
+    const double LN2_HI = 6.93147180369123816490e-01, LN2_LO = 1.90821492927058770002e-10;
+    int e = 0;
+    double m = __builtin_frexp(x, &e);                        // m in [1/2, 1)
+    if (m < 7.07106781186547524401e-01) { m = m * 2.0; e -= 1; }
+    const double s = (m - 1.0) / (m + 1.0), z = s * s;
+    double p = 1.0 / 25.0;
+    for (int k = 23; k >= 1; k -= 2) p = p * z + 1.0 / (double) k;
+    const double lm = (2.0 * s) * p;
+    return (double) e * LN2_HI + ((double) e * LN2_LO + lm);
+}
 template <uint32_t KT>
 __global__ void __launch_bounds__(64) prep_k(const float * __restrict__ qg, const float * __restrict__ k,
                                              const float * __restrict__ v, const float * __restrict__ qn,
                                              const float * __restrict__ kn, const int32_t * __restrict__ pos,
                                              float * __restrict__ q, float * __restrict__ gate, char * kc, char * vc, int p0,
-                                             int Hq, int Hkv, int D, int n_rot, float freq_base, float eps, int ldq, int ldk,
+                                             int Hq, int Hkv, int D, int n_rot, double ln_base, float eps, int ldq, int ldk,
                                              int ldv, kv_view pg, mrope_view mr) {
     const int t = blockIdx.y, b = blockIdx.x, i = threadIdx.x;
     const bool live = 4 * i < D;                               // dead lanes form whole 8-lane groups (D % 32 == 0)
@@ -188,10 +260,9 @@ __global__ void __launch_bounds__(64) prep_k(const float * __restrict__ qg, cons
     for (int sl = 0; sl < 2; ++sl) {
         const int jj = i + 64 * sl;
         if (jj < half) {
-            const float inv = (float) pow((double) freq_base, -2.0 * (double) jj / (double) n_rot);
+            const float inv = (float) det_exp(((-2.0 * (double) jj) / (double) n_rot) * ln_base);
             const float theta = (float) pair_pos(jj) * inv;
-            tc[sl] = (float) cos((double) theta);
-            tsn[sl] = (float) sin((double) theta);
+            det_sincos((double) theta, tc[sl], tsn[sl]);
         }
     }
 #pragma unroll
@@ -308,8 +379,9 @@ int launch_prep(const p1a_kv & c, const float * qg, const float * k, const float
     const kv_view pg = view_of(c);
     const dim3 grid(Hq + 2 * c.Hkv, T);
     char * kc = (char *) c.k, * vc = (char *) c.v;
+    const double ln_base = det_log((double) freq_base);
 #define P1A_PREP(KT_) prep_k<KT_><<<grid, 64, 0, s>>>(qg, k, v, q_norm, k_norm, pos, q, gate, kc, vc, p0, Hq, c.Hkv, c.D, n_rot, \
-                                                      freq_base, eps, ldq, ldk, ldv, pg, mr)
+                                                      ln_base, eps, ldq, ldk, ldv, pg, mr)
     if (c.type == P1A_KV_F16) P1A_PREP(P1A_KV_F16);
     else if (c.type == P1A_KV_Q8_0) P1A_PREP(P1A_KV_Q8_0);
     else P1A_PREP(P1A_KV_Q4_0);

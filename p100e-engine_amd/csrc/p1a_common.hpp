@@ -128,9 +128,11 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
                    float scale, void * scratch, size_t scratch_bytes, hipStream_t s);
 // fold of split partials [rows][NS][D] + (m, l) [rows][NS][2] into out [rows][D] (rows = T * Hq), sigmoid gate fused
 int launch_merge(const float * part_o, const float * part_ml, float * out, const float * gate, int NS, int D, int Hq, int T, hipStream_t s);
-// the library's own split-partial buffers of (current device, stream), grown to at least these sizes; false (nothing
-// reported) when that is not possible now, e.g. the stream is being captured and the buffers would have to grow
+// the library's own buffers for the partials of a key-split prefill on (current device, stream), at least these sizes;
+// false (error set) when that is not possible now, e.g. the stream is being captured and they would have to be allocated
 bool split_scratch(hipStream_t s, size_t bytes_o, size_t bytes_ml, float *& o, float *& ml);
+// bytes of partials a key-split prefill of this shape needs on the current device (0, 0 = one split)
+void prefill_part_need(int T, int p0, int Hq, int D, size_t & bytes_o, size_t & bytes_ml);
 int cu_count();   // compute units of the current device
 int launch_sigmoid_mul(float * x, const float * g, size_t n, hipStream_t s);
 int launch_stream_read(const void * src, size_t bytes, hipStream_t s);   // benchmarks only

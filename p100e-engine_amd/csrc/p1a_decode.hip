@@ -52,13 +52,6 @@ template <uint32_t KT, int D> struct tile_cfg {
     static_assert(HB % 16 == 0, "head row must be a whole number of 16-byte chunks");
 };
 
-#ifdef P1A_TRACE
-// development build only: per-wave phase timestamps (shader clock) in a caller-visible buffer
-__device__ long long * g_trace = nullptr;
-#define TS(i) do { if (g_trace && lane == 0) g_trace[((size_t) blockIdx.x * NWV + wave) * 16 + (i)] = clock64(); } while (0)
-#else
-#define TS(i) do { } while (0)
-#endif
 
 struct dec_params {
     const float * q;
@@ -138,7 +131,6 @@ template <int NR> __device__ __forceinline__ void wait_tiles(int newer) {
 __device__ __forceinline__ int sload_i32(const int32_t * p) {
     return *reinterpret_cast<const __attribute__((address_space(4))) int32_t *>(rfl64((size_t) p));
 }
-__device__ __forceinline__ void wait_scalar(int &) { }
 
 template <uint32_t KT, int D, int NT, int NWV, bool MULTI>
 __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const dec_params P) {
@@ -191,8 +183,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     int pg0_early = 0;
     if (ptab) pg0_early = sload_i32(ptab + idx_early);
     const int p0v = P.pos_rows ? 0 : (P.p0_dev ? *P.p0_dev : P.p0);
-    TS(0);
-
     char * const ks0 = kb0 + wave * C::SLOT_B, * const ks1 = kb1 + wave * C::SLOT_B;
     char * const vs0 = vb0 + wave * C::SLOT_B, * const vs1 = vb1 + wave * C::SLOT_B;
     char * const tab = tabs + wave * C::TAB_B;
@@ -263,9 +253,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         if (tile_start(0) >= n_max) return;
         int pg0 = pg0_early;
         if (ptab && (!first || (tile_start(0) >> P.pg.psh) != idx_early)) pg0 = sload_i32(page_of(tile_start(0)));
-        TS(8);
-        wait_scalar(pg0);
-        TS(9);
         off0 = tile_off(tile_start(0), pg0);
 #pragma unroll
         for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ks0, P.kc + off0, tile_start(0), rd);
@@ -285,8 +272,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     }
     request_k0(true);
     request_v0();
-    TS(1);
-
     // Q^T operands: column = query row (token t, head hh of the group), 8 consecutive dims per MFMA slot group. The
     // rows are the same for every wave of the workgroup, so the workgroup scales and rounds them once - every thread its
     // piece - into an f16 table over V slot 1 (rows padded: conflict-free reads), and every lane picks its operands
@@ -321,8 +306,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         }
     }
     __syncthreads();                                          // both copies are done with: tile 1 may be requested
-
-    TS(2);
     f4 o[NT][C::NDT];
     f4 ol[NT];
     float m_run[NT];
@@ -353,8 +336,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         int pgn = 0;
         if (ptab && have_n) pgn = sload_i32(page_of(tn));
         wait_vm_imm<C::NRND>();                               // K of tile t has landed (only its V is younger)
-        if (t == 0) TS(3); else if (t == 3) TS(4);
-        wait_scalar(pgn);
         const size_t on = have_n ? tile_off(tn, pgn) : 0;
         const char * const kn = P.kc + on, * const vn = P.vc + on;
         // ---- S^T = K Q^T ----
@@ -551,8 +532,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         step(ks0, vs0, ks1, vs1, t);
         if (tile_start(t + 1) < n_max) step(ks1, vs1, ks0, vs0, t + 1);
     }
-    TS(5);
-
     // ---- fold the waves of the workgroup (in wave order) and write one partial per (workgroup, head); the 16
     // columns of one MFMA tile at a time, so that a column is merged the same way whatever NT is. A wave parks its
     // accumulators in its own (now idle) slots, dim quarter k in slot array k, and (m, l) in its table ----
@@ -574,7 +553,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
             }
         }
         __syncthreads();
-        if (r == 0) TS(6);
         // 32 lanes per column: the factors of a column (one per wave; a wave that saw no visible key parked zeros and
         // gets the factor 0) are worked out once per lane and serve all the dims the lane folds
         constexpr int LPC = 32;
@@ -623,7 +601,6 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         }
     }
     }   // streams of this workgroup
-    TS(7);
 }
 
 // ---- generic path: any D % 32 == 0 (<= 512), any GQA, every type; one wave per (split stream, q head, row) ----
@@ -820,11 +797,6 @@ bool mfma_ok(const p1a_kv & c, int GQA) {
     return true;
 }
 
-int env_int(const char * name, int dflt) {
-    const char * e = getenv(name);
-    return e && *e ? atoi(e) : dflt;
-}
-
 dec_plan make_plan(const p1a_kv & c, int Hq, int rows_per_group, int nsplit_req, int cus) {
     dec_plan p;
     p.GQA = Hq / c.Hkv;
@@ -860,12 +832,10 @@ void finish_plan(dec_plan & p) {
 // as bring it back there (a power of two that divides nsplit; measured: 8 slots of unequal depth 89 -> 80 us at 2,
 // 91 us at 4 - fewer, longer workgroups balance worse). The partials do not depend on it.
 int streams_per_wg(const dec_plan & p, int Hkv, int T, int cus) {
-    static const int env = env_int("P1A_DEC_SPW", 0);         // development A/B knob
     const long long wgs = (long long) p.nsplit * Hkv * ((T + p.RG - 1) / p.RG);
     const int per_round = (p.NW == 8 ? 1 : 2) * cus;
     int spw = 1;
     while (spw * 2 <= p.nsplit && p.nsplit % (spw * 2) == 0 && wgs / spw > 4LL * per_round) spw *= 2;
-    if (env > 0 && p.nsplit % env == 0) spw = env;
     return spw;
 }
 
@@ -946,9 +916,6 @@ int launch_merge(const float * part_o, const float * part_ml, float * out, const
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
-#ifdef P1A_TRACE
-extern "C" void p1a_set_trace(long long * buf) { (void) hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &buf, sizeof buf); }
-#endif
 
 // Benchmarks only: a plain streaming read. Workgroup b reads one contiguous span, every lane 16 bytes at a time with four
 // loads in flight; the sum is kept so that the loads cannot be dropped, and stored nowhere (it never equals the sentinel

@@ -64,12 +64,6 @@ template <int D> struct pf_lay {
     static constexpr int v_hi(int ps) { return v_lo(ps) + 8 * VB; }
 };
 
-#ifdef P1A_TRACE
-__device__ long long * g_pf_trace = nullptr;   // development build only: per-workgroup phase cycle totals
-#define PT(i) do { __builtin_amdgcn_sched_barrier(0); const long long t_ = clock64(); acc_t[i] += t_ - last_t; last_t = t_; __builtin_amdgcn_sched_barrier(0); } while (0)
-#else
-#define PT(i) do { } while (0)
-#endif
 
 struct pf_params {
     const float * q;
@@ -546,10 +540,6 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
     // (the first step overwrites K(0) while it runs; every wave has to be done reading it)
     if constexpr (DMA) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-#ifdef P1A_TRACE
-    long long acc_t[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    long long last_t = clock64();
-#endif
     for (int it = 0; it < ntiles; ++it) {
         const int k0 = tile_of(it) * BN;
         char * const st_cur = lds + (it & 1) * L::STAGE_B;             // holds K(it) (done with) and V(it)
@@ -580,8 +570,6 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
                 for (int dt = 0; dt < HD; ++dt) o[0][dt][i] *= alpha;
             }
         }
-        PT(0);
-
         // ---- stream 1: S^T(it+1) on the matrix pipe; stream 2: P^T(it) = exp2(S^T(it) - m) on the vector pipe ----
         // Written step by step, one MFMA per step, with a scheduling fence after each: the LDS read of the K fragment
         // PF_K steps ahead, the MFMA, and a slice of the softmax that fits in the MFMA's shadow.
@@ -625,8 +613,6 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-
-        PT(2);
         // ---- O^T += V^T(it) P^T: set-up. V(it) has been in LDS since the last barrier, so its first fragments are asked
         // for ahead of the exchange: their latency hides behind it ----
         // Slot e of lane half g in k-step ps is key 32 (ps / 2) + 8 (ps % 2) + 4 g + e (e < 4), or that + 16 for e - 4
@@ -650,7 +636,6 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         for (int ps = 0; ps < BN / 16; ++ps) *reinterpret_cast<h8 *>(px_own + (ps * 64 + lane) * 16) = pb[ps];
         if (g == 0) ax_own[c] = alpha;
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        PT(6);
         // ---- stream 1: O^T += V^T(it) P^T on the matrix pipe; stream 2: masking and row maximum of S^T(it+1) (and K(it+2),
         // V(it+1) -> f16 tiles in LDS when they are staged through registers) ----
         {
@@ -690,7 +675,6 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
         }
 
         mloc = row_max(mloc);
-        PT(3);
         // ---- raw loads of K(it+3), V(it+2): one whole step to arrive. Issued back to back: a vector memory instruction
         // holds the wave for as long as the CU's address path needs for it, wherever it is placed ----
         if constexpr (DMA) {
@@ -704,15 +688,10 @@ __global__ void __launch_bounds__(NTHR, 1) prefill_k(const pf_params P) {
             if constexpr (SVL) { sk = load_sblk(P.kc, tile_of(it + 3), gb_k); sv = load_sblk(P.vc, tile_of(it + 2), gb_prev); }
             gb_prev = gb_k;
         }
-        PT(4);
         // LDS stores retired, then the barrier (without the global-memory fence of __syncthreads())
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        PT(5);
     }
 
-#ifdef P1A_TRACE
-    if (g_pf_trace && tid == 0) for (int i = 0; i < 8; ++i) g_pf_trace[(size_t) blockIdx.x * 8 + i] = acc_t[i];
-#endif
     // ---- epilogue: the pair swaps denominators, then each wave normalises, gates and stores its half of the dims of
     // all 64 rows. Lane (row c, half g) holds dims 32 dt + 8 (i / 4) + 4 g + (i % 4) of tile dt ----
     if (g == 0) ax_own[c] = ol[0];
@@ -802,11 +781,10 @@ template <uint32_t KT, int D>
 int launch_pf(const pf_params & P, hipStream_t s) {
     const bool grouped = !P.pg.pt || P.pg.psh >= 4;
     if constexpr (KT == P1A_KV_F16 && D == 256) {
-        static const bool no_dma = getenv("P1A_PF_NODMA") && atoi(getenv("P1A_PF_NODMA"));   // development A/B switch
         // (rows of whole 16-byte units at 16-byte aligned addresses: what a 16-byte load per lane needs)
         // and whole 16-key groups that can be read: always inside a page; inside a contiguous cache when it holds them
         const bool groups_ok = P.pg.pt || ((P.p0 + P.T - 1) | 15) < P.n_rows;
-        if (grouped && !no_dma && groups_ok && P.pg.rowb % 16 == 0 && P.pg.rowb * 16 < (1ull << 32)) return launch_pf_g<KT, D, true, true>(P, s);
+        if (grouped && groups_ok && P.pg.rowb % 16 == 0 && P.pg.rowb * 16 < (1ull << 32)) return launch_pf_g<KT, D, true, true>(P, s);
     }
     return grouped ? launch_pf_g<KT, D, true>(P, s) : launch_pf_g<KT, D, false>(P, s);
 }
@@ -878,6 +856,11 @@ int prefill_key_splits(int T, int p0, int Hq, int cus) {
 }
 size_t prefill_part_bytes_o(int T, int Hq, int D, int nks) { return nks > 1 ? (size_t) T * Hq * nks * D * 4 : 0; }
 size_t prefill_part_bytes_ml(int T, int Hq, int nks) { return nks > 1 ? (((size_t) T * Hq * nks * 2 * 4) + 255) & ~(size_t) 255 : 0; }
+void prefill_part_need(int T, int p0, int Hq, int D, size_t & bytes_o, size_t & bytes_ml) {
+    const int nks = prefill_key_splits(T, p0, Hq, cu_count());
+    bytes_o = prefill_part_bytes_o(T, Hq, D, nks);
+    bytes_ml = prefill_part_bytes_ml(T, Hq, nks);
+}
 
 // bytes of the f16 staging copy of the first n positions (K and V)
 // (rows rounded up to whole 16-key groups: the attention kernel fetches whole groups)
@@ -897,18 +880,16 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
     // the caller's scratch: first the f16 staging copy of a quantized cache (when it fits), then the split partials (when
     // they fit behind it); partials that do not fit go to the library's own per-stream buffers
     const int n = p0 + T;
-    static const bool no_stage = getenv("P1A_PF_NOSTAGE") && atoi(getenv("P1A_PF_NOSTAGE"));   // development A/B switch
-    static const int ks_env = getenv("P1A_PF_SPLIT") ? atoi(getenv("P1A_PF_SPLIT")) : 0;          // development A/B switch
     const bool aligned = scratch && !((uintptr_t) scratch & 255);
-    const bool stage = c.type != P1A_KV_F16 && !no_stage && aligned && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D);
+    const bool stage = c.type != P1A_KV_F16 && aligned && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D);
     const size_t used = stage ? (prefill_stage_bytes(n, c.Hkv, c.D) + 255) & ~(size_t) 255 : 0;
-    int nks = ks_env > 0 ? ks_env : prefill_key_splits(T, p0, Hq, cu_count());
+    const int nks = prefill_key_splits(T, p0, Hq, cu_count());
     if (nks > 1) {
         const size_t bo = prefill_part_bytes_o(T, Hq, c.D, nks), bm = prefill_part_bytes_ml(T, Hq, nks);
         if (aligned && scratch_bytes >= used + bm + bo) {
             P.part_ml = reinterpret_cast<float *>((char *) scratch + used);
             P.part_o = reinterpret_cast<float *>((char *) scratch + used + bm);
-        } else if (!split_scratch(s, bo, bm, P.part_o, P.part_ml)) nks = 1;   // (no room anywhere, e.g. during stream capture)
+        } else if (!split_scratch(s, bo, bm, P.part_o, P.part_ml)) return P1A_E_SCRATCH;   // (the split count fixes the result bits: never fewer splits for want of room)
     }
     P.nks = nks;
     auto finish = [&](int rc) {
@@ -941,9 +922,6 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
 
 }   // namespace p1a
 
-#ifdef P1A_TRACE
-extern "C" void p1a_set_pf_trace(long long * buf) { (void) hipMemcpyToSymbol(HIP_SYMBOL(p1a::g_pf_trace), &buf, sizeof buf); }
-#endif
 
 extern "C" size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D) {
     if (T < 1 || p0 < 0 || Hkv < 1 || D < 1) return 0;

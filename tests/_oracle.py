@@ -53,6 +53,10 @@ def lib():
         L.orc_attn_prep.restype = ctypes.c_int
         L.orc_attn_prep_mrope.argtypes = L.orc_attn_prep.argtypes + [ctypes.POINTER(orc_mrope)]
         L.orc_attn_prep_mrope.restype = ctypes.c_int
+        L.orc_prep_inv_freq.argtypes = [ctypes.c_float, ctypes.c_int, ctypes.c_int]
+        L.orc_prep_inv_freq.restype = ctypes.c_double
+        L.orc_prep_sincos.argtypes = [ctypes.c_float, ctypes.POINTER(ctypes.c_float), ctypes.POINTER(ctypes.c_float)]
+        L.orc_prep_sincos.restype = None
         L.orc_a16_quant.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
         L.orc_kv_fill_random.argtypes = [ctypes.POINTER(orc_kv), ctypes.c_int, ctypes.c_int, ctypes.c_uint32]
         L.orc_num_threads.restype = ctypes.c_int

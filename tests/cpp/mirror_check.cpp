@@ -207,6 +207,93 @@ static void test_type(uint32_t type, hipStream_t s) {
         }
         CK(hipFree(qg)); CK(hipFree(kk)); CK(hipFree(vv)); CK(hipFree(wn)); CK(hipFree(g1)); CK(hipFree(g2)); CK(hipFree(dpos)); CK(hipFree(drt));
     }
+    {   // the rest of the surface the reference headers declare: the device-position and v2 entry points, the standalone
+        // gate and gate + a16 emit, the split-count and environment knobs - each against the call it must equal
+        const int sq = 1, T = 3, p0 = 5000;
+        int32_t * dp0; CK(hipMalloc(&dp0, 16));
+        const int32_t hp0 = p0;
+        CK(hipMemcpy(dp0, &hp0, 4, hipMemcpyHostToDevice));
+        const size_t ob = (size_t) T * Hq * D * 4;
+        F::attn_decode(q, cc[sq], o1, T, p0, Hq, scale, s);
+        CK(hipStreamSynchronize(s));
+        const auto base = bytes_of(o1, ob);
+        const bool d1 = F::attn_decode_dev(q, paged(sq), o2, T, dp0, MAXP * PS, Hq, scale, s);
+        CK(hipStreamSynchronize(s));
+        check("attn_decode_dev == attn_decode", d1 && bytes_of(o2, ob) == base);
+        CK(hipMemset(o2, 0, ob));
+        const bool d2 = F::attn_decode2(q, cc[sq], o2, T, p0, nullptr, Hq, scale, s);
+        CK(hipStreamSynchronize(s));
+        const bool d2a = d2 && bytes_of(o2, ob) == base;
+        CK(hipMemset(o2, 0, ob));
+        const bool d3 = F::attn_decode2(q, paged(sq), o2, T, 0, dp0, Hq, scale, s);
+        CK(hipStreamSynchronize(s));
+        check("attn_decode2 (host and device p0) == attn_decode", d2a && d3 && bytes_of(o2, ob) == base);
+        {   // kv_append_dev writes the rows kv_append writes
+            F::kv_cache a1 = F::kv_alloc(type, 64, Hkv, D), a2 = F::kv_alloc(type, 64, Hkv, D);
+            float * ks = dev_rand((size_t) T * Hkv * D, 1.0f), * vs = dev_rand((size_t) T * Hkv * D, 1.0f);
+            const int32_t h7 = 7;
+            CK(hipMemcpy(dp0, &h7, 4, hipMemcpyHostToDevice));
+            F::kv_append(a1, ks, vs, 7, T, s);
+            F::kv_append_dev(a2, ks, vs, dp0, T, s);
+            CK(hipStreamSynchronize(s));
+            check("kv_append_dev == kv_append", bytes_of(a1.k, 64 * rowb) == bytes_of(a2.k, 64 * rowb) && bytes_of(a1.v, 64 * rowb) == bytes_of(a2.v, 64 * rowb));
+            F::kv_free(a1); F::kv_free(a2); CK(hipFree(ks)); CK(hipFree(vs));
+        }
+        {   // the fused gate of attn_decode == attn_decode followed by sigmoid_mul; ew_quant(EW_SIGMOID_MUL) writes the same rows
+            float * gt = dev_rand((size_t) T * Hq * D, 1.0f), * o3;
+            void * qb; CK(hipMalloc(&qb, p1a_a16_bytes(T, Hq * D))); CK(hipMalloc(&o3, ob));
+            F::attn_decode(q, cc[sq], o2, T, p0, Hq, scale, s, gt);
+            F::sigmoid_mul(o1, gt, (int64_t) T * Hq * D, s);      // o1 holds the ungated rows
+            CK(hipStreamSynchronize(s));
+            const auto fused = bytes_of(o2, ob);
+            check("attn_decode with gate == attn_decode + sigmoid_mul", fused == bytes_of(o1, ob));
+            CK(hipMemcpy(o1, base.data(), ob, hipMemcpyHostToDevice));
+            const bool e1 = F::ew_quant(F::EW_SIGMOID_MUL, o1, gt, o3, qb, T, Hq * D, s);
+            CK(hipStreamSynchronize(s));
+            check("ew_quant(EW_SIGMOID_MUL) rows == the fused gate's", e1 && bytes_of(o3, ob) == fused);
+            CK(hipFree(gt)); CK(hipFree(qb)); CK(hipFree(o3));
+        }
+        {   // attn_prefill_variant is attn_prefill; the split-count knobs; the environment re-read
+            const int Tp = 70, pp = 900;
+            const bool v1 = F::attn_prefill(q, cc[sq], o1, Tp, pp, Hq, scale, s), v2 = F::attn_prefill_variant(q, cc[sq], o2, Tp, pp, Hq, scale, s, 2);
+            CK(hipStreamSynchronize(s));
+            check("attn_prefill_variant == attn_prefill", v1 && v2 && bytes_of(o1, (size_t) Tp * Hq * D * 4) == bytes_of(o2, (size_t) Tp * Hq * D * 4));
+            const int n0 = F::attn_dec2_nsplit(Hkv);
+            F::attn_dec2_set_nsplit(16);
+            const bool k1 = F::attn_dec2_nsplit(Hkv) == 16;
+            F::attn_dec2_set_nsplit(0);
+            const bool k2 = F::attn_dec2_nsplit(Hkv) == n0 && n0 >= 8;
+            (void) F::attn_dec2_reload_env();
+            setenv("P1A_DEC_SPLIT", "24", 1);
+            const bool r1 = F::attn_dec2_reload_env(), k3 = F::attn_dec2_nsplit(Hkv) == 24, r2 = F::attn_dec2_reload_env();
+            unsetenv("P1A_DEC_SPLIT");
+            const bool r3 = F::attn_dec2_reload_env(), k4 = F::attn_dec2_nsplit(Hkv) == n0;
+            check("attn_dec2_nsplit / set_nsplit / reload_env", k1 && k2 && r1 && k3 && !r2 && r3 && k4);
+        }
+        {   // kv_append_rows: rows of two sequences at their own positions == kv_append into each
+            int32_t * dpos, * drt; CK(hipMalloc(&dpos, 64)); CK(hipMalloc(&drt, 64));
+            const int32_t hp[2] = {len[0], len[2]}, hr[2] = {0 * MAXP, 2 * MAXP};
+            CK(hipMemcpy(dpos, hp, 8, hipMemcpyHostToDevice)); CK(hipMemcpy(drt, hr, 8, hipMemcpyHostToDevice));
+            float * ks = dev_rand((size_t) 2 * Hkv * D, 1.0f), * vs = dev_rand((size_t) 2 * Hkv * D, 1.0f);
+            F::kv_cache pc = paged(0);
+            pc.pt = dtab; pc.rtab = drt;
+            const bool a = F::kv_append_rows(pc, ks, vs, dpos, 2, s);
+            F::kv_append(cc[0], ks, vs, len[0], 1, s);
+            F::kv_append(cc[2], ks + (size_t) Hkv * D, vs + (size_t) Hkv * D, len[2], 1, s);
+            CK(hipStreamSynchronize(s));
+            auto hpool = bytes_of(pool, (size_t) NP * pstride);
+            bool ok = a;
+            for (int i = 0; i < 2; ++i) {
+                const int sq2 = i ? 2 : 0, p = len[sq2];
+                const size_t o = (size_t) tabs[(size_t) sq2 * MAXP + (p >> PSH)] * pstride + (size_t) 2 * PS * rowb + (size_t) (p & (PS - 1)) * rowb;
+                auto hk = bytes_of((char *) cc[sq2].k + (size_t) p * rowb, rowb), hv = bytes_of((char *) cc[sq2].v + (size_t) p * rowb, rowb);
+                ok = ok && !memcmp(hk.data(), hpool.data() + o, rowb) && !memcmp(hv.data(), hpool.data() + o + PS * rowb, rowb);
+            }
+            check("kv_append_rows == kv_append per sequence", ok);
+            CK(hipFree(dpos)); CK(hipFree(drt)); CK(hipFree(ks)); CK(hipFree(vs));
+        }
+        CK(hipFree(dp0));
+    }
     {   // a refusal launches nothing and leaves out untouched
         CK(hipMemset(o1, 0x5a, 4096));
         const bool r = F::attn_decode(q, cc[0], o1, 1, 10, Hq + 1, scale, s);

@@ -55,3 +55,25 @@ def test_cpp_mirror_header_compiles():
     r = subprocess.run(["/opt/rocm/bin/hipcc", "-std=c++17", "-fsyntax-only", "-x", "c++", "-I" + os.path.join(ROOT, "include"),
                         "-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__", "-"], input=src, capture_output=True, text=True)
     assert r.returncode == 0, r.stderr[-2000:]
+
+
+def test_reload_env(p1a):
+    """attn_dec2_reload_env (src/fast/attn_dec2.cuh:21): true exactly when the baked-in switch changed"""
+    import os
+    Hkv = 2
+    old = os.environ.pop("P1A_DEC_SPLIT", None)
+    try:
+        p1a.reload_env()
+        n0 = p1a.get_nsplit(Hkv)
+        assert not p1a.reload_env()
+        os.environ["P1A_DEC_SPLIT"] = "24"
+        assert p1a.reload_env()
+        assert p1a.get_nsplit(Hkv) == 24
+        assert not p1a.reload_env()
+        del os.environ["P1A_DEC_SPLIT"]
+        assert p1a.reload_env()
+        assert p1a.get_nsplit(Hkv) == n0
+    finally:
+        if old is not None:
+            os.environ["P1A_DEC_SPLIT"] = old
+        p1a.reload_env()

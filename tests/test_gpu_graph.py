@@ -145,3 +145,88 @@ def test_two_streams_and_two_host_threads(p1a):
     for t in th: t.start()
     for t in th: t.join()
     assert not bad, bad
+
+
+def test_captured_graph_survives_larger_calls_on_its_stream(p1a):
+    """the engine's normal flow: a decode graph captured after the warm-up, then eager work on the same stream that needs
+    the library's buffers at other sizes - a 32-row decode, a key-split prefill without caller scratch, a decode of another
+    head shape (more scratch than the first footprint) - and then the graph again: the buffers it holds are still there,
+    so it gives the bits of the eager call"""
+    Hq, Hkv, D, psh, n = 12, 2, 256, 6, 5000
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, psh, [n], seed=121)
+    c = pool.dev_seq(0)
+    q, _, _, gate = I.qkv(122, 1, 4, Hq, Hkv, D)
+    dq, dg = dev(q), dev(gate)
+    pos = dev(np.array([n - 4], np.int32))
+    s = torch.cuda.Stream()
+    out = torch.zeros((4, Hq, D), device="cuda")
+    big = Pool(p1a, O.KV_F16, 32, 2, 256, 6, [600], seed=123)           # GQA 16: another head shape, a larger footprint
+    qb, _, _, _ = I.qkv(124, 1, 2, 32, 2, 256)
+    q32, _, _, g32 = I.qkv(125, 1, 32, Hq, Hkv, D)
+    qp, _, _, gp = I.qkv(126, 1, 100, Hq, Hkv, D, f16_inputs=True)
+    assert p1a.prefill_key_splits(100, n - 100, Hq) > 1
+    with torch.cuda.stream(s):
+        p1a.warmup(8, Hq, Hkv, D)
+        eager = torch.zeros((4, Hq, D), device="cuda")
+        p1a.attn_decode_dev(dq, c, eager, 4, pos, 0, Hq, 1 / 16, gate=dg)
+        s.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            p1a.attn_decode_dev(dq, c, out, 4, pos, 0, Hq, 1 / 16, gate=dg)
+        graph.replay()
+        s.synchronize()
+        assert torch.equal(out, eager)
+        # eager calls that need other buffers
+        o32 = torch.zeros((32, Hq, D), device="cuda")
+        p1a.attn_decode(dev(q32), c, o32, 32, n - 32, Hq, 1 / 16, gate=dev(g32))
+        op = torch.zeros((100, Hq, D), device="cuda")
+        p1a.attn_prefill(dev(qp), c, op, 100, n - 100, Hq, 1 / 16, gate=dev(gp))
+        ob = torch.zeros((2, 32, 256), device="cuda")
+        p1a.attn_decode(dev(qb), big.dev_seq(0), ob, 2, 598, 32, 1 / 16)
+        s.synchronize()
+        check(o32.cpu().numpy(), O.attn_rows(pool.host_seq(0), q32, (n - 32 + np.arange(32)).astype(np.int32), Hq, 1 / 16, gate=g32), "32 rows")
+        for rep in range(3):
+            out.zero_()
+            graph.replay()
+            # (the program's own eager work between replays)
+            p1a.attn_decode(dev(qb), big.dev_seq(0), ob, 2, 598, 32, 1 / 16)
+            s.synchronize()
+            assert torch.equal(out, eager), rep
+
+
+def test_captured_key_split_prefill_is_refused_or_exact(p1a):
+    """the key-split count fixes the result bits, so it never depends on whether the stream is being captured: without the
+    library's partial buffers the captured call is refused; after p1a_warmup_prefill it gives the eager bits"""
+    Hq, Hkv, D, psh, n, T = 12, 2, 256, 6, 6000, 100
+    pool = Pool(p1a, O.KV_Q8_0, Hq, Hkv, D, psh, [n], seed=127)
+    c = pool.dev_seq(0)
+    qp, _, _, gp = I.qkv(128, 1, T, Hq, Hkv, D, f16_inputs=True)
+    dq, dg = dev(qp), dev(gp)
+    assert p1a.prefill_key_splits(T, n - T, Hq) > 1
+    eager = torch.zeros((T, Hq, D), device="cuda")
+    p1a.attn_prefill(dq, c, eager, T, n - T, Hq, 1 / 16, gate=dg)
+    torch.cuda.synchronize()
+    s = torch.cuda.Stream()                                            # a stream the library has never seen
+    out = torch.zeros((T, Hq, D), device="cuda")
+    refused = False
+    with torch.cuda.stream(s):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s):
+            try:
+                p1a.attn_prefill(dq, c, out, T, n - T, Hq, 1 / 16, gate=dg)
+            except p1a.P1AError:
+                refused = True
+    assert refused
+    s2 = torch.cuda.Stream()
+    with torch.cuda.stream(s2):
+        p1a.warmup_prefill(T, n - T, Hq, Hkv, D)
+        s2.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=s2):
+            p1a.attn_prefill(dq, c, out, T, n - T, Hq, 1 / 16, gate=dg)
+        for rep in range(2):
+            out.zero_()
+            graph.replay()
+            s2.synchronize()
+            assert torch.equal(out, eager), rep
+

@@ -153,8 +153,7 @@ def test_append_random_case(p1a, case):
 def test_prep_random_case(p1a, case):
     """attn_prep (q | gate split, per-head RMS norm * weight, NEOX rotation of the first n_rot dims, quantizing KV write)
     over random shapes, rotary widths, row strides, positions up to a million, host-position and device-position mode, with
-    and without interleaved M-RoPE: gate and V bytes exact, q within one ulp (two double-precision trigonometry libraries),
-    K bytes equal but for the few codes a last-bit difference of the rotated value moves"""
+    and without interleaved M-RoPE: gate, q, V bytes and K bytes all bit for bit the oracle's"""
     g = I.rng(9300 + case)
     kv_type = TYPES[int(g.integers(3))]
     D = int(g.choice([64, 128, 256]))
@@ -197,10 +196,6 @@ def test_prep_random_case(p1a, case):
                   n_rot, base, 1e-6, ldq=ldq, ldk=ldk, ldv=ldv, mrope=mr_dev)
     torch.cuda.synchronize()
     assert np.array_equal(gate.cpu().numpy(), gate_ref), what
-    qd = q.cpu().numpy()
-    ia, ib = qd.view(np.int32).astype(np.int64), q_ref.view(np.int32).astype(np.int64)
-    ia, ib = np.where(ia < 0, -(ia & 0x7fffffff), ia), np.where(ib < 0, -(ib & 0x7fffffff), ib)
-    assert np.abs(ia - ib).max() <= 1, (what, int(np.abs(ia - ib).max()))
+    assert np.array_equal(q.cpu().numpy().view(np.int32), q_ref.view(np.int32)), what
     assert np.array_equal(c._keep[1].cpu().numpy(), host.v), what
-    kd = c._keep[0].cpu().numpy()
-    assert np.count_nonzero(kd != host.k) <= max(4, kd.size // 5000), (what, int(np.count_nonzero(kd != host.k)))
+    assert np.array_equal(c._keep[0].cpu().numpy(), host.k), what

@@ -237,3 +237,35 @@ def test_mrope_moving_one_stream_moves_only_its_pairs():
         q1, _ = O.attn_prep(c, qg, k, v, qn, kn, np.array([0], np.int32), -1, Hq, n_rot, 1e4, mrope=(mp, (11, 11, 10), sect))
         changed = {j for j in range(32) if q1[0, 0, j] != q0[0, 0, j] or q1[0, 0, j + 32] != q0[0, 0, j + 32]}
         assert changed == {j for j in range(32) if streams[j] == name}
+
+
+def test_rotary_recipes_against_numpy_float64():
+    """the oracle's power / cosine / sine are IEEE double recipes in a fixed order (no math library, so the GPU kernel can
+    reproduce every bit); here they are held against numpy's float64 functions: base^(-2j/n) to 32 ulps of double (e^(x ln b)
+    carries |x| roundings of x; the value is used rounded to fp32, 2^29 times coarser), the
+    fp32 cosine and sine of an fp32 angle equal to the rounded float64 value except for rare last-bit roundings"""
+    import ctypes
+    L = O.lib()
+    for base in (1e7, 1e4, 5e5, 1e6, 2.0, 123456.789):
+        for n_rot in (8, 32, 64, 128, 256):
+            for j in range(n_rot // 2):
+                got = L.orc_prep_inv_freq(base, j, n_rot)
+                want = float(np.float64(np.float32(base)) ** (-2.0 * j / n_rot))
+                assert abs(got - want) <= 32 * np.spacing(want), (base, n_rot, j, got, want)
+    g = np.random.default_rng(5)
+    angles = np.concatenate([
+        g.uniform(0, 7, 20000), g.uniform(0, 3e5, 20000), g.uniform(0, 2.0 ** 29, 5000), np.arange(0, 64) * (np.pi / 4),
+        np.arange(1, 4000) * (np.pi / 2), [0.0, 1e-30, 1e-8, 262143.0, 1e6],
+    ]).astype(np.float32)
+    c, s = ctypes.c_float(), ctypes.c_float()
+    off = 0
+    for th in angles:
+        L.orc_prep_sincos(float(th), ctypes.byref(c), ctypes.byref(s))
+        wc, ws = np.float32(np.cos(np.float64(th))), np.float32(np.sin(np.float64(th)))
+        for got, want in ((np.float32(c.value), wc), (np.float32(s.value), ws)):
+            if got != want:
+                off += 1
+                assert abs(np.float64(got) - np.float64(want)) <= np.spacing(np.abs(want)) , (th, got, want)
+    assert off <= 4, off          # (a float64 result within a few 2^-53 of an fp32 rounding boundary may round the other way)
+    L.orc_prep_sincos(0.0, ctypes.byref(c), ctypes.byref(s))
+    assert c.value == 1.0 and s.value == 0.0
