@@ -86,9 +86,8 @@ def test_prefill_in_the_fold_tests_input_regime(p1a, kv_type):
     """peaked softmax (logits carried by seven outlier dims: standard deviation 1.5 to 2, a third of it from one dim) over
     32 K keys through the MFMA prefill and the decode kernel. The
     engine's own bar for f16 products in this regime is max|d| / max|ref| < 3e-2 and rms(d) / rms(ref) < 1e-2
-    (tests/fast_attn_fold_test.cu:81-82); this path accumulates in fp32 and is held to a bar ten times tighter here:
-    max|d| <= 3e-3 max|ref| and rel-L2 <= 2e-3. (The 2e-3 / 1e-3 of the benchmark configurations belongs to their
-    RMS-normed inputs, whose logits have a standard deviation of 1; the error of an f16 logit grows with its size.)"""
+    (tests/fast_attn_fold_test.cu:81-82); this path accumulates in fp32 and is held to its own bar here as well:
+    max|d| <= 2e-3 max(1, max|ref|) and rel-L2 <= 1e-3."""
     hq, hkv, p0, T = 12, 2, 32768, 512
     n = p0 + T
     k = fold_fill(n * hkv * D, 1000, 1.0, D).reshape(n, hkv, D)
@@ -111,15 +110,14 @@ def test_prefill_in_the_fold_tests_input_regime(p1a, kv_type):
     got = out.cpu().numpy()
     ma, rl = I.errors(got, ref)
     mr = float(np.abs(ref).max())
-    print(f"[parity] fold-regime prefill type {kv_type}: logit std {logit_std:.2f}, max|d|/max|ref| {ma / mr:.2e}, rel_l2 {rl:.2e}, "
-          f"path bar (2e-3 max|ref|, 1e-3) {'held' if ma <= 2e-3 * max(1, mr) and rl <= 1e-3 else 'not held'}")
+    print(f"[parity] fold-regime prefill type {kv_type}: logit std {logit_std:.2f}, max|ref| {mr:.2f}, max_abs {ma:.2e}, rel_l2 {rl:.2e}")
     assert np.isfinite(got).all() and logit_std > 1.3
-    assert ma <= 3e-3 * mr and rl <= 2e-3, (ma / mr, rl)
+    assert ma <= 2e-3 * max(1.0, mr) and rl <= 1e-3, (ma, mr, rl)
     rows = np.arange(0, T, 61)
     dec = torch.zeros((len(rows), hq, D), device="cuda")
     for i, t in enumerate(rows):
         p1a.attn_decode(dev(q[t:t + 1]), c, dec[i:i + 1], 1, p0 + int(t), hq, 1 / 16)
     torch.cuda.synchronize()
     ma, rl = I.errors(dec.cpu().numpy(), ref[rows])
-    print(f"[parity] fold-regime decode type {kv_type}: max|d|/max|ref| {ma / mr:.2e}, rel_l2 {rl:.2e}")
-    assert ma <= 3e-3 * mr and rl <= 2e-3, (ma / mr, rl)
+    print(f"[parity] fold-regime decode type {kv_type}: max_abs {ma:.2e}, rel_l2 {rl:.2e}")
+    assert ma <= 2e-3 * max(1.0, mr) and rl <= 1e-3, (ma, mr, rl)
