@@ -145,6 +145,20 @@ int p1a_attn_decode(const float *q, const p1a_kv *c, float *out, const float *ga
 int p1a_attn_decode_a16(const float *q, const p1a_kv *c, float *out, const float *gate, void *qbuf, int T, int p0,
                         const int32_t *p0_dev, const int32_t *pos_rows, int rows_per_seq, int Hq, float scale,
                         void *stream);
+/*
+ * p1a_attn_decode_a16 for callers that cannot allocate (code under hipGraph capture on a stream the library has not seen,
+ * tight serving loops, harnesses that forbid hipMalloc): NO COUNTERPART IN THE REFERENCE. Same arguments, same kernels,
+ * same result bits, but the split partials live in a fixed array in device memory (P1A_NOALLOC_SCRATCH_BYTES, one copy per
+ * GPU, held until the process ends) instead of the library's per-stream buffers, and the call never allocates or frees
+ * anything. A call whose partials do not fit (T * Hq * splits * (D + 2) * 4 bytes; 8 rows of the 24 / 4 / 256 shape fit for
+ * every KV type: 64 split streams for q8_0 / q4_0, 128 for f16) is refused with P1A_E_SCRATCH. Every call on one GPU shares that GPU's array: calls that overlap on one GPU
+ * (two streams, two threads) race - serialise them. The array's address is looked up on the first call per device (or by
+ * p1a_warmup).
+ */
+#define P1A_NOALLOC_SCRATCH_BYTES (32u << 20)
+int p1a_attn_decode_noalloc(const float *q, const p1a_kv *c, float *out, const float *gate, void *qbuf, int T, int p0,
+                            const int32_t *p0_dev, const int32_t *pos_rows, int rows_per_seq, int Hq, float scale,
+                            void *stream);
 /* bytes of the a16 buffer of T rows of n values (n % 32 == 0): T * n/32 * (16 + 1) half2 */
 size_t p1a_a16_bytes(int T, int n);
 /*

@@ -7,7 +7,7 @@ import os
 KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
-    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_kv_fill_random", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
+    "p1a_kv_row_bytes", "p1a_kv_append", "p1a_kv_fill_random", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_attn_decode_noalloc", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_reload_env", "p1a_warmup_prefill", "p1a_bench_decode_split_only", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
     "p1a_version",
     # include/p1a_pool.h
@@ -69,6 +69,8 @@ def lib():
     L.p1a_attn_prep_mrope.argtypes = [vp] * 8 + [kvp, i32, i32, i32, i32, f32, f32, i32, i32, i32, vp, i32, i32, i32, i32, i32, vp]
     L.p1a_attn_decode_a16.restype = i32
     L.p1a_attn_decode_a16.argtypes = [vp, kvp, vp, vp, vp, i32, i32, vp, vp, i32, i32, f32, vp]
+    L.p1a_attn_decode_noalloc.restype = i32
+    L.p1a_attn_decode_noalloc.argtypes = [vp, kvp, vp, vp, vp, i32, i32, vp, vp, i32, i32, f32, vp]
     L.p1a_a16_bytes.restype = sz
     L.p1a_a16_bytes.argtypes = [i32, i32]
     L.p1a_ew_quant.restype = i32

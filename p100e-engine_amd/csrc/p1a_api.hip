@@ -8,6 +8,11 @@
 #include <cstring>
 #include <mutex>
 
+// Split scratch of the allocation-free decode entry point (p1a_attn_decode_noalloc): a fixed array in device memory,
+// one copy per GPU, held until the process ends. In host code the array's NAME is only a handle: its device address is
+// asked for once per device with hipGetSymbolAddress and only that address is ever handed to kernels.
+static __device__ __align__(256) unsigned char scratch[P1A_NOALLOC_SCRATCH_BYTES];
+
 namespace p1a {
 
 static thread_local char g_err[256] = "";
@@ -29,10 +34,10 @@ namespace {
 // old one only for later calls - the old one stays allocated (g_retired) until p1a_release(). Nothing is allocated
 // while the stream is being captured. The partials of a key-split prefill have a pair of their own.
 struct bufpair { float * o = nullptr; float * ml = nullptr; size_t cap_o = 0, cap_ml = 0; };
-struct scratch { int dev = -1; hipStream_t s = nullptr; bufpair dec, pf; };
+struct stream_bufs { int dev = -1; hipStream_t s = nullptr; bufpair dec, pf; };
 constexpr int MAX_SCR = 64;
 constexpr int MAX_RETIRED = 1024;
-scratch g_scr[MAX_SCR];
+stream_bufs g_scr[MAX_SCR];
 int g_nscr = 0;
 struct retired { int dev; void * p; };
 retired g_retired[MAX_RETIRED];
@@ -41,8 +46,29 @@ std::mutex g_mu;
 int g_nsplit_override = 0;
 int g_env_split = -1;   // P1A_DEC_SPLIT as last read (-1 = not read yet)
 int g_cus[16] = {0};
+constexpr int MAX_DEV = 64;
+void * g_static_scratch[MAX_DEV] = {nullptr};   // device address of `scratch` on each device (nullptr = not asked for yet)
 
 }   // namespace
+
+// the device address of the static split scratch on the CURRENT device (resolved on the first call per device), or
+// nullptr with the error set
+void * static_scratch() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEV) { set_error("p1a_attn_decode_noalloc: no current device"); return nullptr; }
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_static_scratch[dev]) {
+        void * ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(::scratch));
+        if (e != hipSuccess || !ptr) {
+            (void) hipGetLastError();
+            set_error("p1a_attn_decode_noalloc: hipGetSymbolAddress failed (%s)", hipGetErrorString(e));
+            return nullptr;
+        }
+        g_static_scratch[dev] = ptr;
+    }
+    return g_static_scratch[dev];
+}
 
 int cu_count() {
     int dev = 0;
@@ -61,7 +87,7 @@ bufpair * scratch_for(hipStream_t s, which_buf w, size_t need_o, size_t need_ml,
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return nullptr;
     std::lock_guard<std::mutex> lk(g_mu);
-    scratch * e = nullptr;
+    stream_bufs * e = nullptr;
     for (int i = 0; i < g_nscr; ++i) if (g_scr[i].dev == dev && g_scr[i].s == s) e = &g_scr[i];
     if (!e) {
         if (g_nscr == MAX_SCR) { if (!quiet) set_error("too many (device, stream) pairs"); return nullptr; }
@@ -273,6 +299,15 @@ int p1a_attn_decode_a16(const float * q, const p1a_kv * c, float * out, const fl
     return decode_call(q, c, out, gate, qbuf, T, p0, p0_dev, pos_rows, rows_per_seq, Hq, scale, false, (hipStream_t) stream);
 }
 
+int p1a_attn_decode_noalloc(const float * q, const p1a_kv * c, float * out, const float * gate, void * qbuf, int T, int p0,
+                            const int32_t * p0_dev, const int32_t * pos_rows, int rows_per_seq, int Hq, float scale,
+                            void * stream) {
+    void * ptr = static_scratch();
+    if (!ptr) return P1A_E_SCRATCH;
+    return decode_call(q, c, out, gate, qbuf, T, p0, p0_dev, pos_rows, rows_per_seq, Hq, scale, false, (hipStream_t) stream,
+                       ptr, P1A_NOALLOC_SCRATCH_BYTES);
+}
+
 int p1a_bench_decode_split_only(const float * q, const p1a_kv * c, float * out, int T, int p0, const int32_t * p0_dev,
                                 const int32_t * pos_rows, int rows_per_seq, int Hq, float scale, void * stream) {
     return decode_call(q, c, out, nullptr, nullptr, T, p0, p0_dev, pos_rows, rows_per_seq, Hq, scale, true, (hipStream_t) stream);
@@ -282,6 +317,7 @@ int p1a_warmup(int rows, int Hq, int Hkv, int D, void * stream) {
     if (rows < 1 || rows > P1A_MAX_ROWS || Hq < 1 || Hkv < 1 || Hq % Hkv || D < 32) { set_error("p1a_warmup: bad shape"); return P1A_E_ARG; }
     size_t need_o, need_ml;
     decode_footprint(Hq, Hkv, D, need_o, need_ml);
+    (void) static_scratch();   // set-up time: the allocation-free entry point then has nothing left to resolve on this device
     return scratch_for((hipStream_t) stream, BUF_DECODE, need_o, need_ml) ? P1A_OK : P1A_E_SCRATCH;
 }
 
@@ -338,7 +374,7 @@ void p1a_release(void) {
         (void) hipDeviceSynchronize();
         for (bufpair * b : {&g_scr[i].dec, &g_scr[i].pf})
             if (b->o) { (void) hipFree(b->o); (void) hipFree(b->ml); }
-        g_scr[i] = scratch{};
+        g_scr[i] = stream_bufs{};
     }
     g_nscr = 0;
     for (int i = 0; i < g_nretired; ++i) {
