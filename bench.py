@@ -4,8 +4,9 @@
 Workload (N = 1): configs[1] of the baseline description - 27B-shape decode, batch 1, one full-attention layer: 24 q heads / 4 kv
 heads, head_dim 256, context 32768, q8_0 KV in 256-token pages scattered by a random permutation page table, fused
 sigmoid gate. A "step" is one p1a_attn_decode call (split-K kernel + merge) on inputs resident in HBM. The K timed
-steps are captured once into a hipGraph (the engine replays its decode step as a graph as well) and walk over several
-distinct KV pools, so that consecutive steps do not find their 71 MB of KV in the 256 MB Infinity Cache.
+steps are captured once into a hipGraph (the engine replays its decode step as a graph as well) and walk over the KV of
+8 full-attention layers of one sequence (the engine's pool layout: each layer its own K / V bytes, one page table per
+sequence), so that consecutive steps do not find their 71 MB of KV in the 256 MB Infinity Cache.
 
 Prints ONE JSON line: metric / value (GB/s of algorithmic KV bytes) plus `roofline` and `cpu_baseline` objects, and
 secondary measurements (same-pool rate, verify, batched decode, prefill, append) under `extra`.
@@ -24,6 +25,29 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def build_layers(p1a, torch, kv_type, Hkv, D, psh, n_ctx, n_layers, seed):
+    """ONE sequence of n_ctx tokens in a paged pool of n_layers full-attention layers, the engine's layout
+    [page][layer][K | V][2^psh][rowb]: every layer has its own K / V bytes, all layers share the sequence's page table (a random
+    permutation). Returns the per-layer descriptors; K/V are N(0,1), K RMS-normed per head, written through the library's
+    own quantize-on-append."""
+    ps = 1 << psh
+    n_pages = (n_ctx + ps - 1) // ps
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    tab = torch.randperm(n_pages, generator=g, device="cuda").to(torch.int32)
+    rowb = p1a.kv_row_bytes(kv_type, Hkv, D)
+    pool = torch.zeros(n_pages * n_layers * 2 * ps * rowb, dtype=torch.uint8, device="cuda")
+    layers = [p1a.KVCache.paged(kv_type, Hkv, D, psh, n_pages, tab, n_pages, n_layers=n_layers, layer=l, pool=pool) for l in range(n_layers)]
+    for c in layers:
+        for a in range(0, n_ctx, 4096):
+            T = min(4096, n_ctx - a)
+            k = torch.randn((T, Hkv, D), generator=g, device="cuda")
+            k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + 1e-6)
+            v = torch.randn((T, Hkv, D), generator=g, device="cuda")
+            p1a.kv_append(c, k, v, a, T)
+    torch.cuda.synchronize()
+    return layers, n_pages
 
 
 def build_pool(p1a, torch, kv_type, Hq, Hkv, D, psh, n_ctx, n_seq, seed, lens=None):
@@ -305,14 +329,16 @@ def host_view(torch, kv, ppseq, slot, Hkv, D, psh, kv_type):
     return h.view(pt=np.ascontiguousarray(tabs[slot * ppseq:(slot + 1) * ppseq]))
 
 
-def cpu_baseline(torch, kv, ppseq, slot, q, gate, out_gpu, Hq, Hkv, D, psh, n_ctx, scale):
+def cpu_baseline(torch, kv, layer, n_layers, q, gate, out_gpu, Hq, Hkv, D, psh, n_ctx, scale):
     """The CPU oracle (fp32 restatement of the reference's attention kernel, OpenMP over heads) on a bounded sample of
     the same workload: the decode step the GPU timed last - same pool bytes, same page table, same q and gate - repeated
     for about 10 s; its result is the check of the GPU's timed output."""
     import numpy as np
     import _inputs as I
     import _oracle as O
-    hv = host_view(torch, kv, ppseq, slot, Hkv, D, psh, O.KV_Q8_0)
+    pool = kv.pool.cpu().numpy()
+    tab = kv.pt.cpu().numpy()
+    hv = O.HostKV.paged(O.KV_Q8_0, Hkv, D, psh, len(tab), tab, len(tab), n_layers=n_layers, layer=layer, pool=pool)
     hq, hg = q.cpu().numpy(), gate.cpu().numpy()
     pos = np.array([n_ctx - 1], np.int32)
     ref = O.attn_rows(hv, hq, pos, Hq, scale, gate=hg)
@@ -327,7 +353,7 @@ def cpu_baseline(torch, kv, ppseq, slot, q, gate, out_gpu, Hq, Hkv, D, psh, n_ct
     model, ncpu = host_cpu()
     bytes_ = 2 * n_ctx * O.row_bytes(O.KV_Q8_0, Hkv, D)
     return {"value": round(bytes_ * reps / dt / 1e9, 2), "unit": "GB/s", "cores": int(O.lib().orc_num_threads()), "kind": "port",
-            "sample": f"{reps} full decode steps (1 row, ctx {n_ctx}, q8_0, the pool and page table of the GPU's last timed step) of "
+            "sample": f"{reps} full decode steps (1 row, ctx {n_ctx}, q8_0, the layer and page table of the GPU's last timed step) of "
                       f"the C oracle with OpenMP, {dt:.1f} s",
             "cpu_model": model, "nproc": ncpu,
             "gpu_output_check": {"max_abs": float(f"{ma:.3e}"), "rel_l2": float(f"{rl:.3e}"), "tol": [I.MAX_ABS_TOL, I.REL_L2_TOL],
@@ -399,8 +425,8 @@ def main():
         return
     rowb = p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
     step_bytes = 2 * n_ctx * rowb                                          # K + V of the visible positions
-    n_pools = 8                                                            # 8 x 71 MB > 256 MB Infinity Cache
-    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, n_ctx, n_pools, seed=1234)
+    n_pools = 8                                                            # 8 layers x 71 MB > 256 MB Infinity Cache
+    slots, ppseq = build_layers(p1a, torch, p1a.KV_Q8_0, Hkv, D, psh, n_ctx, n_pools, seed=1234)
     g = torch.Generator(device="cuda").manual_seed(99)
     q = torch.randn((1, Hq, D), generator=g, device="cuda")
     q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + 1e-6)
@@ -409,7 +435,6 @@ def main():
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         p1a.warmup(32, Hq, Hkv, D)
-    slots = [kv.slot(s, ppseq) for s in range(n_pools)]
 
     def step(i):
         return lambda: p1a.attn_decode(q, slots[i % n_pools], out, 1, n_ctx - 1, Hq, scale, gate=gate)
@@ -438,14 +463,14 @@ def main():
         "n_gpus": 1, "steps": K, "warmup": W, "ms_per_step": round(sec * 1e3, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "q8_0 KV -> f16 MFMA, f32 accumulate", "data": "synthetic",
         "config": {"workload": "configs[1]: decode 24/4 heads, head_dim 256, ctx 32768, q8_0, 256-token pages, random page table",
-                   "kv_bytes_per_step": step_bytes, "pools_rotated": n_pools,
+                   "kv_bytes_per_step": step_bytes, "layers_rotated": n_pools,
                    "launch": f"hipGraph of K steps, replayed {REPLAYS} times, median replay"},
         "replay_ms_per_step": [round(x * 1e3, 5) for x in samples],
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": "dec_mfma_k<q8_0, 256, 1, 8>",
                      "kernel_us": round(sec_kernel * 1e6, 2),
                      "note": "achieved = algorithmic KV bytes of one launch (2 * ctx * 1088 B) / average duration of the "
-                             "split-K kernel, event-timed on its stream over a graph of K launches on rotating pools (median of "
+                             "split-K kernel, event-timed on its stream over a graph of K launches walking the 8 layers (median of "
                              f"{REPLAYS} replays); traffic = HBM bytes per launch read from the committed rocprofv3 counter summary "
                              "(profiles/decode_q8_0_32k_traffic.json), not measured in this run"},
         "extra": {"same_pool_GBs": sec_same and round(step_bytes / sec_same / 1e9, 1), "same_pool_us": sec_same and round(sec_same * 1e6, 2),
@@ -468,8 +493,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if not args.no_cpu:
-        res["cpu_baseline"] = cpu_baseline(torch, kv, ppseq, (K - 1) % n_pools, q, gate, out_timed, Hq, Hkv, D, psh, n_ctx, scale)
-    del kv, slots
+        res["cpu_baseline"] = cpu_baseline(torch, slots[(K - 1) % n_pools], (K - 1) % n_pools, n_pools, q, gate, out_timed, Hq, Hkv, D, psh, n_ctx, scale)
+    del slots
     if not args.no_extra:
         top = {}
         res["extra"].update(extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, not args.no_cpu))

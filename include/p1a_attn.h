@@ -222,7 +222,7 @@ int p1a_reload_env(void);
 int p1a_bench_decode_split_only(const float *q, const p1a_kv *c, float *out, int T, int p0, const int32_t *p0_dev,
                                 const int32_t *pos_rows, int rows_per_seq, int Hq, float scale, void *stream);
 /* Benchmarks only (no counterpart in the reference): a plain read of `bytes` bytes of device memory (16 bytes per lane,
- * one contiguous span per workgroup, nothing computed) - the time the memory system needs for a launch of that size,
+ * one contiguous span per workgroup, four workgroups per compute unit, nothing computed) - the time the memory system needs for a launch of that size,
  * to set a decode launch of the same number of KV bytes against. bytes is rounded down to a multiple of 16. */
 int p1a_bench_stream_read(const void *src, size_t bytes, void *stream);
 /* free every scratch buffer of the current process (after synchronising the devices that own them); graphs captured

@@ -89,6 +89,15 @@ __device__ __forceinline__ u2 deq4(uint32_t w, h2 d01, h2 d23) {
     return u2{__builtin_bit_cast(uint32_t, (a - off) * d01), __builtin_bit_cast(uint32_t, (b - off) * d23)};
 }
 
+// q * scale rounded to fp32, then to f16: two roundings, spelled out. Left to itself the compiler turns (half) (q * s) into
+// a fused multiply-convert (one rounding) in some places and into a multiply and a convert in others, and two kernel
+// variants could then disagree in the last bit of a Q operand - rows must not depend on the variant that ran.
+__device__ __forceinline__ half_t scale_to_half(float q, float s) {
+    float p = q * s;
+    asm volatile("" : "+v"(p));
+    return (half_t) p;
+}
+
 // the maximum over the four lanes that share (lane & 15): the two 16-lane rows of each half, then the two halves
 __device__ __forceinline__ float max_over_groups(float m) { return max_swap32(max_swap16(m)); }
 
@@ -285,7 +294,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);          // (columns past the live ones: zero operands)
         if (col < R) a = *reinterpret_cast<const float4 *>(kb1 + (size_t) i * 16);
         const float s = P.qscale;
-        *reinterpret_cast<h4 *>(qt + col * C::QRS + d * 2) = h4{(half_t) (a.x * s), (half_t) (a.y * s), (half_t) (a.z * s), (half_t) (a.w * s)};
+        *reinterpret_cast<h4 *>(qt + col * C::QRS + d * 2) = h4{scale_to_half(a.x, s), scale_to_half(a.y, s), scale_to_half(a.z, s), scale_to_half(a.w, s)};
     }
     __syncthreads();
     h8 qf[QLDS ? 1 : NT][QLDS ? 1 : C::NMF];
@@ -918,8 +927,10 @@ int launch_merge(const float * part_o, const float * part_ml, float * out, const
 
 
 // Benchmarks only: a plain streaming read. Workgroup b reads one contiguous span, every lane 16 bytes at a time with four
-// loads in flight; the sum is kept so that the loads cannot be dropped, and stored nowhere (it never equals the sentinel
-// for the inputs a benchmark uses; one float of static device memory takes it if it ever does).
+// loads in flight, four workgroups of 512 threads per compute unit (measured on a 71 MB read inside a graph: 13.4 us
+// with one workgroup per unit, 11.5 with two, 11.25 with four; deeper per-lane queues instead of more waves do worse);
+// the sum is kept so that the loads cannot be dropped, and stored nowhere (it never equals the sentinel for the inputs a
+// benchmark uses; one float of static device memory takes it if it ever does).
 __device__ float g_stream_read_sink;
 __global__ void __launch_bounds__(512) stream_read_k(const f4 * __restrict__ p, size_t n16) {
     const size_t per = n16 / gridDim.x;
@@ -939,7 +950,7 @@ __global__ void __launch_bounds__(512) stream_read_k(const f4 * __restrict__ p, 
 int launch_stream_read(const void * src, size_t bytes, hipStream_t s) {
     int dev = 0, cus = 256;
     if (hipGetDevice(&dev) == hipSuccess) (void) hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    stream_read_k<<<cus > 0 ? cus : 256, 512, 0, s>>>(reinterpret_cast<const f4 *>(src), bytes / 16);
+    stream_read_k<<<4 * (cus > 0 ? cus : 256), 512, 0, s>>>(reinterpret_cast<const f4 *>(src), bytes / 16);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
