@@ -189,38 +189,9 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
         sec = time_graph(torch, stream, [lambda: p1a.attn_prep(qg4, kc, vc, w_q, w_k, pos4, q4, g4, c, p0, 4, Hq, 64, 1e7, 1e-6)] * 20, 2)
     ex["prep_4rows_q8_0_us"] = round(sec * 1e6, 2)
     del kv, c, q, gate, out
-    # configs[3]: MTP verify, 4 sequences x 4 rows, q4_0, ctx 65536
-    n4 = 65536
-    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q4_0, Hq, Hkv, D, psh, n4, 4, seed=22)
-    pos = torch.tensor([n4 - 4 + t for _ in range(4) for t in range(4)], dtype=torch.int32, device="cuda")
-    rt = torch.tensor([s * ppseq for s in range(4) for _ in range(4)], dtype=torch.int32, device="cuda")
-    q = normed((16, Hq, D)).half().float()
-    out = torch.empty((16, Hq, D), device="cuda")
-    cr = kv.with_rows(rt)
-    with torch.cuda.stream(stream):
-        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 16, pos, Hq, scale, rows_per_seq=4)] * 20, 2)
-    vb = 4 * n4 * 2 * p1a.kv_row_bytes(p1a.KV_Q4_0, Hkv, D)
-    ex["verify_4x4_q4_0_64K_us"] = round(sec * 1e6, 2)
-    ex["verify_GBs"] = round(vb / sec / 1e9, 1)
-    del kv, cr
+    ex.update(verify_config(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     ex.update(mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale))
-    # configs[2]: 8 slots, one row each, ctx log-uniform in [1024, 32768], q8_0, one shared pool
-    rs = torch.Generator().manual_seed(8)
-    lens = [int(math.exp(float(torch.empty(1).uniform_(math.log(1024), math.log(32768), generator=rs)))) for _ in range(8)]
-    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, 32768, 8, seed=23, lens=lens)
-    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32, device="cuda")
-    rt = torch.tensor([s * ppseq for s in range(8)], dtype=torch.int32, device="cuda")
-    q = normed((8, Hq, D))
-    gate = torch.randn((8, Hq * D), generator=g, device="cuda")
-    out = torch.empty((8, Hq, D), device="cuda")
-    cr = kv.with_rows(rt)
-    with torch.cuda.stream(stream):
-        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 8, pos, Hq, scale, gate=gate)] * 20, 2)
-    bb = sum(lens) * 2 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
-    ex["batched_8slots_q8_0_us"] = round(sec * 1e6, 2)
-    ex["batched_GBs"] = round(bb / sec / 1e9, 1)
-    ex["batched_ctx"] = lens
-    del kv, cr
+    ex.update(batched_config(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     # the same kernel with enough to stream: 4 sequences of 65536 tokens, one row each, q8_0 (570 MB of KV per call)
     n4 = 65536
     kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, n4, 4, seed=24)
@@ -236,6 +207,47 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
     ex["decode_4x64K_q8_0_us"] = round(sec * 1e6, 2)
     ex["decode_4x64K_GBs"] = round(lb / sec / 1e9, 1)
     return ex
+
+
+def verify_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
+    """configs[3]: MTP verify, 4 sequences x 4 rows (causal inside the block), q4_0, ctx 65536, each sequence's KV read once"""
+    n4 = 65536
+    g = torch.Generator(device="cuda").manual_seed(6)
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q4_0, Hq, Hkv, D, psh, n4, 4, seed=22)
+    pos = torch.tensor([n4 - 4 + t for _ in range(4) for t in range(4)], dtype=torch.int32, device="cuda")
+    rt = torch.tensor([s * ppseq for s in range(4) for _ in range(4)], dtype=torch.int32, device="cuda")
+    q = torch.randn((16, Hq, D), generator=g, device="cuda")
+    q = (q * torch.rsqrt((q * q).mean(-1, keepdim=True) + 1e-6)).half().float()
+    out = torch.empty((16, Hq, D), device="cuda")
+    cr = kv.with_rows(rt)
+    with torch.cuda.stream(stream):
+        p1a.warmup(32, Hq, Hkv, D)
+        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 16, pos, Hq, scale, rows_per_seq=4)] * reps, 2)
+        sec_k = time_graph(torch, stream, [lambda: p1a.bench_decode_split_only(q, cr, out, 16, 0, Hq, scale, pos=pos, rows_per_seq=4)] * reps, 2)
+    vb = 4 * n4 * 2 * p1a.kv_row_bytes(p1a.KV_Q4_0, Hkv, D)
+    return {"verify_4x4_q4_0_64K_us": round(sec * 1e6, 2), "verify_GBs": round(vb / sec / 1e9, 1),
+            "verify_kernel_us": round(sec_k * 1e6, 2), "verify_kernel_frac_of_hbm_peak": round(vb / sec_k / 1e9 / HBM_PEAK_GBS, 4)}
+
+
+def batched_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
+    """configs[2]: 8 slots, one row each, ctx log-uniform in [1024, 32768], q8_0, one shared pool"""
+    import math
+    g = torch.Generator(device="cuda").manual_seed(9)
+    rs = torch.Generator().manual_seed(8)
+    lens = [int(math.exp(float(torch.empty(1).uniform_(math.log(1024), math.log(32768), generator=rs)))) for _ in range(8)]
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, 32768, 8, seed=23, lens=lens)
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32, device="cuda")
+    rt = torch.tensor([s * ppseq for s in range(8)], dtype=torch.int32, device="cuda")
+    q = torch.randn((8, Hq, D), generator=g, device="cuda")
+    q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + 1e-6)
+    gate = torch.randn((8, Hq * D), generator=g, device="cuda")
+    out = torch.empty((8, Hq, D), device="cuda")
+    cr = kv.with_rows(rt)
+    with torch.cuda.stream(stream):
+        p1a.warmup(32, Hq, Hkv, D)
+        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 8, pos, Hq, scale, gate=gate)] * reps, 2)
+    bb = sum(lens) * 2 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
+    return {"batched_8slots_q8_0_us": round(sec * 1e6, 2), "batched_GBs": round(bb / sec / 1e9, 1), "batched_ctx": lens}
 
 
 def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, steps=30):
@@ -399,6 +411,11 @@ def main():
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the chunked-prefill configuration (T = 4096 after 28672 tokens, q8_0) a few times and print its "
                          "time: a short program for rocprofv3 counter passes over prefill_k")
+    ap.add_argument("--verify-only", action="store_true",
+                    help="run only the MTP-verify configuration (4 sequences x 4 rows, q4_0, ctx 65536) a few times and print its "
+                         "time: a short program for rocprofv3 counter passes over dec_mfma_k<q4_0, 256, 2, 8>")
+    ap.add_argument("--batched-only", action="store_true",
+                    help="run only the batched-decode configuration (8 slots of unequal depth, q8_0) a few times and print its time")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is measured on ONE GPU only (no collectives are part of it); run with --gpus 1", file=sys.stderr)
@@ -422,6 +439,12 @@ def main():
         sec = time_eager(torch, lambda: p1a.attn_prefill(qp, c, op, T, p0, Hq, scale, gate=gp, scratch=scr), reps=3, warmup=1)
         flop = 4.0 * D * Hq * (p0 * T + T * (T + 1) / 2)
         print(json.dumps({"prefill_T4096_p28672_q8_0_ms": round(sec * 1e3, 4), "TFLOPs": round(flop / sec / 1e12, 1)}))
+        return
+    if args.verify_only:
+        print(json.dumps(verify_config(p1a, torch, torch.cuda.Stream(), Hq, Hkv, D, psh, scale, reps=10)))
+        return
+    if args.batched_only:
+        print(json.dumps(batched_config(p1a, torch, torch.cuda.Stream(), Hq, Hkv, D, psh, scale, reps=10)))
         return
     rowb = p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
     step_bytes = 2 * n_ctx * rowb                                          # K + V of the visible positions

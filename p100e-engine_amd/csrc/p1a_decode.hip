@@ -222,6 +222,19 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     // "nothing outstanding", and placed after the requests such a wait would also wait for the tiles.
 #pragma unroll
     for (int r = 0; r < NT; ++r) asm volatile("" : "+v"(plim[r]));
+    // A workgroup none of whose streams holds a visible key (a short sequence in a batch: stream s is empty once s units
+    // cover the sequence) writes the empty partials its streams would have ended with and is done.
+    if (split * U >= n_max) {
+        for (int i = threadIdx.x; i < R * spw; i += NWV * 64) {
+            const int col = i % R, sw = i / R;
+            const int t = row_of(col), hh = col - t * P.GQA;
+            const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) hg * P.GQA + hh;
+            float * pm = P.part_ml + (row * P.nsplit + split + sw * nwgs) * 2;
+            pm[0] = NEG_INF;
+            pm[1] = 0.f;
+        }
+        return;
+    }
     const size_t head_off = (size_t) hk * C::HB;
     const int rowb = (int) P.pg.rowb;
 
@@ -545,7 +558,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
     // columns of one MFMA tile at a time, so that a column is merged the same way whatever NT is. A wave parks its
     // accumulators in its own (now idle) slots, dim quarter k in slot array k, and (m, l) in its table ----
     constexpr int QD = D / 4;                                 // dims per quarter
-    char * const st[4] = {kb0, kb1, vb0, vb1};
+    auto st = [&](int k) -> char * { return k == 0 ? kb0 : k == 1 ? kb1 : k == 2 ? vb0 : vb1; };
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         const int Rr = min(16, R - 16 * r);                  // live columns of this tile
@@ -553,7 +566,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
         if (c < Rr) {
 #pragma unroll
             for (int j = 0; j < C::NDT; ++j) {
-                float * dst = reinterpret_cast<float *>(st[j / (C::NDT / 4)] + wave * C::SLOT_B);
+                float * dst = reinterpret_cast<float *>(st(j / (C::NDT / 4)) + wave * C::SLOT_B);
                 *reinterpret_cast<f4 *>(dst + c * C::QDP + 16 * (j % (C::NDT / 4)) + 4 * g) = o[r][j];
             }
             if (g == 0) {
@@ -589,7 +602,7 @@ __global__ void __launch_bounds__(NWV * 64, NWV == 4 ? 2 : 1) dec_mfma_k(const d
 #pragma unroll
             for (int d4 = dl; d4 < D / 4; d4 += LPC) {
                 const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
-                const char * sbase = qtr == 0 ? kb0 : qtr == 1 ? kb1 : qtr == 2 ? vb0 : vb1;
+                const char * sbase = st(qtr);
                 f4 aw[NWV];
 #pragma unroll
                 for (int w = 0; w < NWV; ++w)
@@ -702,15 +715,20 @@ __global__ void __launch_bounds__(256) dec_generic_k(const gen_params P) {
 // out[row][d] = sum_s 2^(m_s - M) O_s[d] / sum_s 2^(m_s - M) l_s; empty streams (m = -inf or l = 0) are skipped.
 // One wave per (row, 32 dims): lane = (slice of the splits, 4 dims); slice k folds splits k, k + 8, ... in order and
 // the 8 slices are then added in order, so the result depends on nothing but the partials.
+// pos_rows / U (optional): row t of a batched call sits at position pos_rows[t] and its split stream s holds keys only when
+// s units of U positions do not cover the sequence yet - the streams past that are known to be empty and are not fetched.
 __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o, const float * __restrict__ part_ml,
-                                              float * __restrict__ out, const float * __restrict__ gate, int NS, int D,
-                                              void * qbuf, int Hq, int T) {
+                                              float * __restrict__ out, const float * __restrict__ gate, int NS_all, int D,
+                                              void * qbuf, int Hq, int T, const int32_t * __restrict__ pos_rows, int U) {
     __shared__ f4 sacc[8][8];
     __shared__ float sden[8];
     const size_t row = blockIdx.x;
+    const int NS_row = NS_all;                                // (the row stride of the partials)
+    int NS = NS_all;
+    if (pos_rows && U > 0) NS = min(NS_all, pos_rows[row / Hq] / U + 1);
     const int tid = threadIdx.x, q4 = tid & 7, sl = tid >> 3;
     const int d = blockIdx.y * 32 + q4 * 4;
-    const float * ml = part_ml + row * NS * 2;
+    const float * ml = part_ml + row * NS_row * 2;
     constexpr int CH = 8;                                     // splits of a slice fetched together
     // the gate depends on nothing here: its load rides along with the first batch of partials
     f4 gt = {0.f, 0.f, 0.f, 0.f};
@@ -725,7 +743,7 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
         ms[k] = NEG_INF; ls[k] = 0.f; a[k] = f4{0.f, 0.f, 0.f, 0.f};
         if (s < NS) {
             ms[k] = ml[2 * s]; ls[k] = ml[2 * s + 1];
-            a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS + s) * D + d);
+            a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS_row + s) * D + d);
         }
     }
     // the maximum over all splits: this slice's (its first batch is in registers already; later batches re-read the pairs),
@@ -745,7 +763,7 @@ __global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o,
                 ms[k] = NEG_INF; ls[k] = 0.f;
                 if (s < NS) {
                     ms[k] = ml[2 * s]; ls[k] = ml[2 * s + 1];
-                    a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS + s) * D + d);
+                    a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS_row + s) * D + d);
                 }
             }
         }
@@ -916,12 +934,13 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
         rc = hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
     }
     if (rc != P1A_OK || a.skip_merge) return rc;
-    merge_k<<<dim3(a.T * a.Hq, c.D / 32), 64, 0, s>>>(a.part_o, a.part_ml, a.out, a.gate, pl.NS, c.D, a.qbuf, a.Hq, a.T);
+    merge_k<<<dim3(a.T * a.Hq, c.D / 32), 64, 0, s>>>(a.part_o, a.part_ml, a.out, a.gate, pl.NS, c.D, a.qbuf, a.Hq, a.T,
+                                                       pl.mfma ? a.pos_rows : nullptr, 32 * pl.NW);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
 int launch_merge(const float * part_o, const float * part_ml, float * out, const float * gate, int NS, int D, int Hq, int T, hipStream_t s) {
-    merge_k<<<dim3((unsigned) T * Hq, D / 32), 64, 0, s>>>(part_o, part_ml, out, gate, NS, D, nullptr, Hq, T);
+    merge_k<<<dim3((unsigned) T * Hq, D / 32), 64, 0, s>>>(part_o, part_ml, out, gate, NS, D, nullptr, Hq, T, nullptr, 0);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
