@@ -713,88 +713,87 @@ __global__ void __launch_bounds__(256) dec_generic_k(const gen_params P) {
 
 // ---- merge of the split partials, in a fixed order, with the fused sigmoid gate ----
 // out[row][d] = sum_s 2^(m_s - M) O_s[d] / sum_s 2^(m_s - M) l_s; empty streams (m = -inf or l = 0) are skipped.
-// One wave per (row, 32 dims): lane = (slice of the splits, 4 dims); slice k folds splits k, k + 8, ... in order and
-// the 8 slices are then added in order, so the result depends on nothing but the partials.
+// One workgroup of 256 threads per (row, 128 dims): thread = (slice of the splits, 4 dims); slice k folds splits k, k + 8,
+// ... in order and the 8 slices are then added in order, so the result depends on nothing but the partials. A wave holds
+// two slices, so each of its loads covers two contiguous half-rows of 512 bytes. The (m, l) pairs are fetched once per
+// wave - lane i brings the pair of split i - and handed round by lane shuffles; the maximum is a wave reduction.
 // pos_rows / U (optional): row t of a batched call sits at position pos_rows[t] and its split stream s holds keys only when
 // s units of U positions do not cover the sequence yet - the streams past that are known to be empty and are not fetched.
-__global__ void __launch_bounds__(64) merge_k(const float * __restrict__ part_o, const float * __restrict__ part_ml,
-                                              float * __restrict__ out, const float * __restrict__ gate, int NS_all, int D,
-                                              void * qbuf, int Hq, int T, const int32_t * __restrict__ pos_rows, int U) {
-    __shared__ f4 sacc[8][8];
+constexpr int MRG_DIMS = 128;
+__global__ void __launch_bounds__(256) merge_k(const float * __restrict__ part_o, const float * __restrict__ part_ml,
+                                               float * __restrict__ out, const float * __restrict__ gate, int NS_all, int D,
+                                               void * qbuf, int Hq, int T, const int32_t * __restrict__ pos_rows, int U) {
+    __shared__ f4 sacc[8][32];
     __shared__ float sden[8];
     const size_t row = blockIdx.x;
     const int NS_row = NS_all;                                // (the row stride of the partials)
     int NS = NS_all;
     if (pos_rows && U > 0) NS = min(NS_all, pos_rows[row / Hq] / U + 1);
-    const int tid = threadIdx.x, q4 = tid & 7, sl = tid >> 3;
-    const int d = blockIdx.y * 32 + q4 * 4;
+    const int tid = threadIdx.x, lane = tid & 63, qd = tid & 31, sl = tid >> 5;
+    const int d = blockIdx.y * MRG_DIMS + qd * 4;
+    const bool live = d < D;
     const float * ml = part_ml + row * NS_row * 2;
     constexpr int CH = 8;                                     // splits of a slice fetched together
     // the gate depends on nothing here: its load rides along with the first batch of partials
     f4 gt = {0.f, 0.f, 0.f, 0.f};
-    if (gate && sl == 0) gt = *reinterpret_cast<const f4 *>(gate + row * D + d);
+    if (gate && sl == 0 && live) gt = *reinterpret_cast<const f4 *>(gate + row * D + d);
+    f4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.f;
+    // the maximum over all splits first: batches of 64 pairs, lane i of every wave the pair of split s0 + i
+    float M = NEG_INF;
+    float2 pr = make_float2(NEG_INF, 0.f);                    // the pair of split `lane` of the first batch
+    if (lane < NS) pr = *reinterpret_cast<const float2 *>(ml + 2 * lane);
     // the first batch of partials (all of them when NS <= 64) is requested before anything is known about the maximum
     f4 a[CH];
-    float ms[CH], ls[CH];
-    float M = NEG_INF;
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
         const int s = sl + 8 * k;
-        ms[k] = NEG_INF; ls[k] = 0.f; a[k] = f4{0.f, 0.f, 0.f, 0.f};
-        if (s < NS) {
-            ms[k] = ml[2 * s]; ls[k] = ml[2 * s + 1];
-            a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS_row + s) * D + d);
-        }
+        a[k] = f4{0.f, 0.f, 0.f, 0.f};
+        if (s < NS && live) a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS_row + s) * D + d);
     }
-    // the maximum over all splits: this slice's (its first batch is in registers already; later batches re-read the pairs),
-    // then over the 8 slices - the lanes that share (lane & 7)
-    for (int s = sl + 8 * CH; s < NS; s += 8) M = fmaxf(M, ml[2 * s]);
+    M = pr.x;
+    for (int s0 = 64; s0 < NS; s0 += 64) if (s0 + lane < NS) M = fmaxf(M, ml[2 * (s0 + lane)]);
 #pragma unroll
-    for (int k = 0; k < CH; ++k) M = fmaxf(M, ms[k]);
-    M = fmaxf(M, __shfl_xor(M, 8));
-    M = max_over_groups(M);
-    f4 num = {0.f, 0.f, 0.f, 0.f};
-    float den = 0.f;
-    for (int s0 = sl; s0 < NS; s0 += 8 * CH) {
-        if (s0 != sl) {
+    for (int w = 1; w < 64; w <<= 1) M = fmaxf(M, __shfl_xor(M, w));
+    for (int s0 = 0; s0 < NS; s0 += 8 * CH) {
+        if (s0) {
+            pr = make_float2(NEG_INF, 0.f);
+            if (s0 + lane < NS) pr = *reinterpret_cast<const float2 *>(ml + 2 * (s0 + lane));
 #pragma unroll
             for (int k = 0; k < CH; ++k) {
-                const int s = s0 + 8 * k;
-                ms[k] = NEG_INF; ls[k] = 0.f;
-                if (s < NS) {
-                    ms[k] = ml[2 * s]; ls[k] = ml[2 * s + 1];
-                    a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS_row + s) * D + d);
-                }
+                const int s = s0 + sl + 8 * k;
+                if (s < NS && live) a[k] = *reinterpret_cast<const f4 *>(part_o + (row * NS_row + s) * D + d);
             }
         }
 #pragma unroll
         for (int k = 0; k < CH; ++k) {
-            if (ms[k] == NEG_INF || ls[k] == 0.f) continue;   // empty stream: its accumulator was never written
-            const float f = __builtin_amdgcn_exp2f(ms[k] - M);
-            den = fmaf(f, ls[k], den);
+            const float msk = __shfl(pr.x, sl + 8 * k), lsk = __shfl(pr.y, sl + 8 * k);
+            if (msk == NEG_INF || lsk == 0.f) continue;       // empty stream: its accumulator was never written
+            const float f = __builtin_amdgcn_exp2f(msk - M);
+            den = fmaf(f, lsk, den);
             num[0] = fmaf(f, a[k][0], num[0]); num[1] = fmaf(f, a[k][1], num[1]);
             num[2] = fmaf(f, a[k][2], num[2]); num[3] = fmaf(f, a[k][3], num[3]);
         }
     }
-    sacc[sl][q4] = num;
-    if (q4 == 0) sden[sl] = den;
+    sacc[sl][qd] = num;
+    if (qd == 0) sden[sl] = den;
     __syncthreads();
     if (sl == 0) {
-        f4 n = sacc[0][q4];
+        f4 n = sacc[0][qd];
         float dn = sden[0];
 #pragma unroll
-        for (int k = 1; k < 8; ++k) { n += sacc[k][q4]; dn += sden[k]; }
+        for (int k = 1; k < 8; ++k) { n += sacc[k][qd]; dn += sden[k]; }
         f4 r = {n[0] / dn, n[1] / dn, n[2] / dn, n[3] / dn};
         if (gate) {
 #pragma unroll
             for (int x = 0; x < 4; ++x) r[x] *= 1.0f / (1.0f + expf(-gt[x]));
         }
-        *reinterpret_cast<f4 *>(out + row * D + d) = r;
-        // the 8 lanes of slice 0 hold one 32-value group of the output row: its a16 activation quantize rides along
-        // (what the engine's ew_quant emits for the output projection, src/fast/fused.cu:478-496)
+        if (live) *reinterpret_cast<f4 *>(out + row * D + d) = r;
+        // 8 consecutive lanes of slice 0 hold one 32-value group of the output row: its a16 activation quantize rides
+        // along (what the engine's ew_quant emits for the output projection, src/fast/fused.cu:478-496)
         if (qbuf) {
             const int t = (int) (row / Hq), h = (int) (row - (size_t) t * Hq);
-            a16_quant8(r, q4, qbuf, t, h * (D >> 5) + (int) blockIdx.y, (Hq * D) >> 5, T, true);
+            a16_quant8(r, qd & 7, qbuf, t, h * (D >> 5) + (d >> 5), (Hq * D) >> 5, T, live);
         }
     }
 }
@@ -934,13 +933,13 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
         rc = hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
     }
     if (rc != P1A_OK || a.skip_merge) return rc;
-    merge_k<<<dim3(a.T * a.Hq, c.D / 32), 64, 0, s>>>(a.part_o, a.part_ml, a.out, a.gate, pl.NS, c.D, a.qbuf, a.Hq, a.T,
+    merge_k<<<dim3(a.T * a.Hq, (c.D + MRG_DIMS - 1) / MRG_DIMS), 256, 0, s>>>(a.part_o, a.part_ml, a.out, a.gate, pl.NS, c.D, a.qbuf, a.Hq, a.T,
                                                        pl.mfma ? a.pos_rows : nullptr, 32 * pl.NW);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
 int launch_merge(const float * part_o, const float * part_ml, float * out, const float * gate, int NS, int D, int Hq, int T, hipStream_t s) {
-    merge_k<<<dim3((unsigned) T * Hq, D / 32), 64, 0, s>>>(part_o, part_ml, out, gate, NS, D, nullptr, Hq, T, nullptr, 0);
+    merge_k<<<dim3((unsigned) T * Hq, (D + MRG_DIMS - 1) / MRG_DIMS), 256, 0, s>>>(part_o, part_ml, out, gate, NS, D, nullptr, Hq, T, nullptr, 0);
     return hipPeekAtLastError() == hipSuccess ? P1A_OK : P1A_E_LAUNCH;
 }
 
