@@ -160,9 +160,15 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
                 "whole p1a_attn_prefill call with caller scratch (the convert-once pass of about 40 us included), median of 5"}
     out_scr = out.clone()
     sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=5)
-    ex["prefill_no_scratch_ms"] = round(sec * 1e3, 4)
+    ex["prefill_no_scratch_ms"] = round(sec * 1e3, 4)                      # (the library's own staging copy: the reference's attn_prefill call site)
     ex["prefill_no_scratch_frac_of_f16_mfma_peak"] = round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)
     ex["prefill_scratch_equals_no_scratch_bits"] = bool(torch.equal(out, out_scr))
+    # neither the caller's scratch nor the library's staging copy: every workgroup dequantizes its own tiles
+    p1a.set_prefill_staging_limit(0)
+    sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=3)
+    p1a.set_prefill_staging_limit(1 << 30)
+    ex["prefill_in_kernel_dequant_ms"] = round(sec * 1e3, 4)
+    ex["prefill_in_kernel_dequant_equals_bits"] = bool(torch.equal(out, out_scr))
     del scr, out_scr
     if cpu:
         top["cpu_prefill"] = cpu_prefill(torch, kv, ppseq, q, gate, out, p0, T, Hq, Hkv, D, psh, scale)

@@ -173,9 +173,12 @@ int p1a_ew_quant(int op, const float *a, const float *b, float *y, void *qbuf, i
  * sequence (page table pt + (rtab ? rtab[0] : 0)); the cache must already hold positions 0..p0+T-1 (append first).
  * fp16 MFMA products with fp32 accumulation; gate as in p1a_attn_decode. `scratch` is optional caller-supplied device
  * memory (256-byte aligned): with at least p1a_attn_prefill_scratch_bytes(...) bytes a q8_0 / q4_0 cache is converted to
- * f16 once per call instead of once per workgroup (same result bits, about 10-35 % less time); with less, or NULL, the
- * kernel converts on the fly. Results do not depend on the scratch passed. Rows of the cache past position p0 + T - 1 may be fetched (never past the end of a page,
- * or of a contiguous cache) but are never weighted, whatever they hold.
+ * f16 once per call instead of once per workgroup (same result bits, about 10-35 % less time). With less, or NULL - the
+ * reference's attn_prefill brings none - the library uses a staging copy of its own, kept per (device, stream) like its
+ * split scratch (allocated and grown outside stream capture only, never freed before p1a_release, at most
+ * p1a_set_prefill_staging_limit bytes, 1 GiB unless set); where it has none the kernel converts on the fly. Results do not
+ * depend on which of the three happened. Rows of the cache past position p0 + T - 1 may be fetched (never past the end of a
+ * page, or of a contiguous cache) but are never weighted, whatever they hold.
  * Replaces attn_prefill (src/fast/attn.cuh:46-50) and attn_fold (src/fast/attn_fold.cuh:19-26).
  */
 int p1a_attn_prefill(const float *q, const p1a_kv *c, float *out, const float *gate, int T, int p0, int Hq,
@@ -193,8 +196,11 @@ size_t p1a_attn_prefill_scratch_bytes(int T, int p0, int Hq, int Hkv, int D);
  * be allocated during stream capture: such a call is refused with P1A_E_SCRATCH unless p1a_warmup_prefill (or an eager
  * call of the shape) came first. */
 int p1a_attn_prefill_key_splits(int T, int p0, int Hq);
+/* Largest f16 staging copy the library keeps per (device, stream) for p1a_attn_prefill calls without caller scratch
+ * (bytes; 0 = never: such calls convert inside the kernel). No counterpart in the reference. */
+void p1a_set_prefill_staging_limit(size_t bytes);
 /* Allocate the library's key-split partial buffers of (current device, stream) for a prefill call of this shape (a no-op
- * for shapes that take one split), so that the call can be captured. No counterpart in the reference, whose attn_fold
+ * for shapes that take one split) and its f16 staging copy (when within the limit), so that the call can be captured. No counterpart in the reference, whose attn_fold
  * takes all scratch from the caller (src/fast/attn_fold.cuh:25-26). */
 int p1a_warmup_prefill(int T, int p0, int Hq, int Hkv, int D, void *stream);
 

@@ -8,7 +8,7 @@ KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 
 EXPORTS = [
     "p1a_kv_row_bytes", "p1a_kv_append", "p1a_kv_fill_random", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_attn_decode_noalloc", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
-    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_reload_env", "p1a_warmup_prefill", "p1a_bench_decode_split_only", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
+    "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_reload_env", "p1a_warmup_prefill", "p1a_set_prefill_staging_limit", "p1a_bench_decode_split_only", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
     "p1a_version",
     # include/p1a_pool.h
     "p1a_pool_create", "p1a_pool_destroy", "p1a_pool_n_pages", "p1a_pool_free_pages", "p1a_pool_max_pages", "p1a_pool_page_bytes",
@@ -95,6 +95,8 @@ def lib():
     L.p1a_set_nsplit.argtypes = [i32]
     L.p1a_reload_env.restype = i32
     L.p1a_reload_env.argtypes = []
+    L.p1a_set_prefill_staging_limit.restype = None
+    L.p1a_set_prefill_staging_limit.argtypes = [sz]
     L.p1a_warmup_prefill.restype = i32
     L.p1a_warmup_prefill.argtypes = [i32, i32, i32, i32, i32, vp]
     L.p1a_bench_decode_split_only.restype = i32
@@ -327,6 +329,10 @@ def set_nsplit(n):
 def reload_env():
     """src/fast/attn_dec2.cuh:21: True when the split-count environment switch changed (captured graphs must be dropped)."""
     return bool(lib().p1a_reload_env())
+
+
+def set_prefill_staging_limit(nbytes):
+    lib().p1a_set_prefill_staging_limit(nbytes)
 
 
 def warmup_prefill(T, p0, Hq, Hkv, D):

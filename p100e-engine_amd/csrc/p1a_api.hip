@@ -34,7 +34,7 @@ namespace {
 // old one only for later calls - the old one stays allocated (g_retired) until p1a_release(). Nothing is allocated
 // while the stream is being captured. The partials of a key-split prefill have a pair of their own.
 struct bufpair { float * o = nullptr; float * ml = nullptr; size_t cap_o = 0, cap_ml = 0; };
-struct stream_bufs { int dev = -1; hipStream_t s = nullptr; bufpair dec, pf; };
+struct stream_bufs { int dev = -1; hipStream_t s = nullptr; bufpair dec, pf; void * stage = nullptr; size_t cap_stage = 0; };
 constexpr int MAX_SCR = 64;
 constexpr int MAX_RETIRED = 1024;
 stream_bufs g_scr[MAX_SCR];
@@ -45,6 +45,7 @@ int g_nretired = 0;
 std::mutex g_mu;
 int g_nsplit_override = 0;
 int g_env_split = -1;   // P1A_DEC_SPLIT as last read (-1 = not read yet)
+size_t g_stage_limit = (size_t) 1 << 30;   // largest f16 staging copy the library keeps per (device, stream); 0 = none
 int g_cus[16] = {0};
 constexpr int MAX_DEV = 64;
 void * g_static_scratch[MAX_DEV] = {nullptr};   // device address of `scratch` on each device (nullptr = not asked for yet)
@@ -206,6 +207,38 @@ bool split_scratch(hipStream_t s, size_t bytes_o, size_t bytes_ml, float *& o, f
     return true;
 }
 
+// The library's own f16 staging copy for a prefill over a quantized cache without caller scratch: a buffer of at least
+// `bytes` bytes of (current device, s), or nullptr when there is none to be had now - over the limit, allocation failed, or
+// the stream is being captured and the buffer would have to be allocated or grown. Never an error: the caller then
+// converts inside the kernel, with the same result bits. Grown in steps (64 MiB granules, at least half as much again),
+// replaced buffers stay allocated until p1a_release() like every buffer a captured graph may hold.
+void * stage_scratch(hipStream_t s, size_t bytes) {
+    int dev = 0;
+    if (!bytes || bytes > g_stage_limit || hipGetDevice(&dev) != hipSuccess) return nullptr;
+    std::lock_guard<std::mutex> lk(g_mu);
+    stream_bufs * e = nullptr;
+    for (int i = 0; i < g_nscr; ++i) if (g_scr[i].dev == dev && g_scr[i].s == s) e = &g_scr[i];
+    if (!e) {
+        if (g_nscr == MAX_SCR) return nullptr;
+        e = &g_scr[g_nscr++];
+        e->dev = dev; e->s = s;
+    }
+    if (bytes <= e->cap_stage) return e->stage;
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    if (s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone) return nullptr;
+    if (e->stage && g_nretired + 1 > MAX_RETIRED) return nullptr;
+    const size_t gran = (size_t) 64 << 20;
+    size_t want = (bytes + gran - 1) / gran * gran;
+    if (want < e->cap_stage + e->cap_stage / 2) want = e->cap_stage + e->cap_stage / 2;
+    if (want > g_stage_limit) want = g_stage_limit;
+    if (want < bytes) want = bytes;
+    void * p = nullptr;
+    if (hipMalloc(&p, want) != hipSuccess) { (void) hipGetLastError(); return nullptr; }
+    if (e->stage) g_retired[g_nretired++] = retired{dev, e->stage};
+    e->stage = p; e->cap_stage = want;
+    return p;
+}
+
 }   // namespace p1a
 
 using namespace p1a;
@@ -325,9 +358,13 @@ int p1a_warmup_prefill(int T, int p0, int Hq, int Hkv, int D, void * stream) {
     if (T < 1 || p0 < 0 || Hq < 1 || Hkv < 1 || Hq % Hkv || D < 32) { set_error("p1a_warmup_prefill: bad shape"); return P1A_E_ARG; }
     size_t bo, bm;
     prefill_part_need(T, p0, Hq, D, bo, bm);
+    // (the f16 staging copy of a quantized cache, when it is within the limit: optional, a call without it converts in the kernel)
+    (void) stage_scratch((hipStream_t) stream, prefill_stage_bytes(p0 + T, Hkv, D));
     if (!bo) return P1A_OK;
     return scratch_for((hipStream_t) stream, BUF_PREFILL, bo, bm) ? P1A_OK : P1A_E_SCRATCH;
 }
+
+void p1a_set_prefill_staging_limit(size_t bytes) { g_stage_limit = bytes; }
 
 int p1a_attn_prefill(const float * q, const p1a_kv * c, float * out, const float * gate, int T, int p0, int Hq,
                      float scale, void * scratch, size_t scratch_bytes, void * stream) {
@@ -374,6 +411,7 @@ void p1a_release(void) {
         (void) hipDeviceSynchronize();
         for (bufpair * b : {&g_scr[i].dec, &g_scr[i].pf})
             if (b->o) { (void) hipFree(b->o); (void) hipFree(b->ml); }
+        if (g_scr[i].stage) (void) hipFree(g_scr[i].stage);
         g_scr[i] = stream_bufs{};
     }
     g_nscr = 0;

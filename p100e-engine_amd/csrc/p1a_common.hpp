@@ -131,6 +131,9 @@ int launch_merge(const float * part_o, const float * part_ml, float * out, const
 // the library's own buffers for the partials of a key-split prefill on (current device, stream), at least these sizes;
 // false (error set) when that is not possible now, e.g. the stream is being captured and they would have to be allocated
 bool split_scratch(hipStream_t s, size_t bytes_o, size_t bytes_ml, float *& o, float *& ml);
+// the library's own f16 staging copy of (current device, stream) for a prefill over a quantized cache (nullptr: none now)
+void * stage_scratch(hipStream_t s, size_t bytes);
+size_t prefill_stage_bytes(int n, int Hkv, int D);
 // bytes of partials a key-split prefill of this shape needs on the current device (0, 0 = one split)
 void prefill_part_need(int T, int p0, int Hq, int D, size_t & bytes_o, size_t & bytes_ml);
 int cu_count();   // compute units of the current device

@@ -881,8 +881,12 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
     // they fit behind it); partials that do not fit go to the library's own per-stream buffers
     const int n = p0 + T;
     const bool aligned = scratch && !((uintptr_t) scratch & 255);
-    const bool stage = c.type != P1A_KV_F16 && aligned && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D);
-    const size_t used = stage ? (prefill_stage_bytes(n, c.Hkv, c.D) + 255) & ~(size_t) 255 : 0;
+    const bool stage_caller = c.type != P1A_KV_F16 && aligned && scratch_bytes >= prefill_stage_bytes(n, c.Hkv, c.D);
+    const size_t used = stage_caller ? (prefill_stage_bytes(n, c.Hkv, c.D) + 255) & ~(size_t) 255 : 0;
+    // no room in the caller's scratch (the reference's attn_prefill brings none): the library's own staging copy, if it has one
+    void * stage_own = nullptr;
+    if (c.type != P1A_KV_F16 && !stage_caller) stage_own = stage_scratch(s, prefill_stage_bytes(n, c.Hkv, c.D));
+    const bool stage = stage_caller || stage_own;
     const int nks = prefill_key_splits(T, p0, Hq, cu_count());
     if (nks > 1) {
         const size_t bo = prefill_part_bytes_o(T, Hq, c.D, nks), bm = prefill_part_bytes_ml(T, Hq, nks);
@@ -903,7 +907,7 @@ int launch_prefill(const p1a_kv & c, const float * q, float * out, const float *
     // would otherwise repeat per 128 query rows. Same tiles, same products, same bits as the direct kernel.
     if (stage) {
         const int n16 = (n + 15) & ~15;
-        char * ko = (char *) scratch, * vo = ko + (size_t) n16 * c.Hkv * c.D * 2;
+        char * ko = (char *) (stage_caller ? scratch : stage_own), * vo = ko + (size_t) n16 * c.Hkv * c.D * 2;
         const long long items = (long long) n * (c.Hkv * c.D / (c.type == P1A_KV_Q8_0 ? 16 : 32));
         const unsigned blocks = (unsigned) ((items + 255) / 256);
         if (c.type == P1A_KV_Q8_0) dq_k<P1A_KV_Q8_0><<<blocks, 256, 0, s>>>(P.kc, P.vc, P.pg, n, c.Hkv, c.D, ko, vo);

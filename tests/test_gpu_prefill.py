@@ -86,12 +86,19 @@ def test_prefill_rows_match_decode(p1a, kv_type):
 @pytest.mark.parametrize("kv_type", [O.KV_Q8_0, O.KV_Q4_0])
 @pytest.mark.parametrize("Hq,Hkv,D,psh", [(12, 2, 256, 5), (8, 2, 128, 4)])
 def test_scratch_variant_gives_the_same_bits(p1a, kv_type, Hq, Hkv, D, psh):
-    """with caller scratch the quantized cache is converted to f16 once and the f16 kernel runs on the copy: same tiles,
-    same products, same bits as the on-the-fly kernel; a scratch that is too small silently takes the direct kernel"""
+    """with scratch - the caller's, or the library's own staging copy when the caller brings none - the quantized cache is
+    converted to f16 once and the f16 kernel runs on the copy: same tiles, same products, same bits as the on-the-fly
+    kernel (staging limit 0); a caller scratch that is too small silently takes the library's copy or the direct kernel"""
     p0, T = 777, 300
     pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [p0 + T, 40], seed=3 + psh, n_layers=2, layer=0)
     q, _, _, gate = I.qkv(70 + D, 1, T, Hq, Hkv, D, f16_inputs=True)
-    a = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16, gate=gate)
+    p1a.set_prefill_staging_limit(0)                                   # no staging copy anywhere: dequantization in the kernel
+    try:
+        direct = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16, gate=gate)
+    finally:
+        p1a.set_prefill_staging_limit(1 << 30)
+    a = run_prefill(p1a, pool.dev_seq(0), q, T, p0, Hq, 1 / 16, gate=gate)      # the library's own staging copy
+    assert np.array_equal(a, direct)
     need = p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D)
     stage = 2 * ((p0 + T + 15) // 16 * 16) * Hkv * D * 2               # whole 16-key groups of f16 rows, K and V
     ks = p1a.prefill_key_splits(T, p0, Hq)                            # (this shape is split over the keys)
