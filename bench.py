@@ -210,6 +210,7 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
     del kvg, cg_
     ex.update(verify_config(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     ex.update(mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale))
+    ex.update(mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, graphed=True))
     ex.update(batched_config(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     # the same kernel with enough to stream: 4 sequences of 65536 tokens, one row each, q8_0 (570 MB of KV per call)
     n4 = 65536
@@ -269,15 +270,24 @@ def batched_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
     return {"batched_8slots_q8_0_us": round(sec * 1e6, 2), "batched_GBs": round(bb / sec / 1e9, 1), "batched_ctx": lens}
 
 
-def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, steps=30):
+def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, steps=30, graphed=False):
     """The verify attention inside a step loop, as the engine's scheduler drives it (accept / rollback per sequence,
     src/sched.cpp:1053-1087 of the reference): 4 sequences of a q4_0 pool at ~64K tokens, every step 1 + 3 draft rows per
     sequence go through attn_prep (norm, rope, quantizing KV write at each row's own position) and one batched
     attn_decode_rows, the host accepts a prefix (each draft right with probability 0.7, seeded) and rolls the rest back.
-    Wall time per step, host bookkeeping and the position upload included."""
+    Wall time per step, host bookkeeping and the position upload included. graphed: the two launches of a step (input prep,
+    batched attention) are captured once into a graph after the warm-up and replayed every step, positions and page tables
+    being read on the device - the way the engine runs its decode step (src/tp_model.cu:1379-1397)."""
     import random
     import time
-    pool = p1a.Pool(p1a.KV_Q4_0, 1, Hkv, D, psh, n_ctx=ctx + 4096, max_slots=n_seq, tokens=n_seq * (ctx + 4096))
+    gs = torch.cuda.Stream()
+    with torch.cuda.stream(gs):
+        res = _mtp_verify_loop(p1a, torch, gs, Hq, Hkv, D, psh, scale, n_seq, ctx, steps, graphed, random, time)
+    return res
+
+
+def _mtp_verify_loop(p1a, torch, gs, Hq, Hkv, D, psh, scale, n_seq, ctx, steps, graphed, random, time):
+    pool = p1a.Pool(p1a.KV_Q4_0, 1, Hkv, D, psh, n_ctx=ctx + 4096, max_slots=n_seq, tokens=n_seq * (ctx + 4096), stream=gs.cuda_stream)
     g = torch.Generator(device="cuda").manual_seed(31)
     ids = [pool.seq_create() for _ in range(n_seq)]
     for i, s in enumerate(ids):
@@ -305,6 +315,19 @@ def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, step
     cr = pool.cache_rows(0)
     rnd = random.Random(7)
     emitted, t_total = 0, 0.0
+
+    def launches():
+        p1a.attn_prep(qg, kx, vx, w, w, pos, q, gate, cr, -1, rows, Hq, 64, 1e7, 1e-6)
+        p1a.attn_decode_rows(q, cr, out, rows, pos, Hq, scale, gate=gate, rows_per_seq=R)
+
+    graph = None
+    if graphed:
+        p1a.warmup(rows, Hq, Hkv, D)
+        pos.copy_(torch.tensor([pool.seq_len(s) - 1 for s in ids for _ in range(R)], dtype=torch.int32))   # (valid rows for the capture)
+        gs.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=gs):
+            launches()
     for step in range(steps + 3):
         t0 = time.perf_counter()
         for i, s in enumerate(ids):
@@ -313,9 +336,11 @@ def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, step
                 pos_h[i * R + t] = n + t
             pool.seq_advance(s, T=R)
         pos.copy_(pos_h, non_blocking=True)
-        p1a.attn_prep(qg, kx, vx, w, w, pos, q, gate, cr, -1, rows, Hq, 64, 1e7, 1e-6)
-        p1a.attn_decode_rows(q, cr, out, rows, pos, Hq, scale, gate=gate, rows_per_seq=R)
-        torch.cuda.synchronize()                            # the engine reads the rows' logits here
+        if graph is not None:
+            graph.replay()
+        else:
+            launches()
+        gs.synchronize()                                    # the engine reads the rows' logits here
         n_out = 0
         for s in ids:
             tokens = [1, 2, 3, 4]
@@ -332,7 +357,8 @@ def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, step
             t_total += dt
             emitted += n_out
     pool.close()
-    return {"mtp_verify_step_us": round(t_total / steps * 1e6, 1), "mtp_tokens_per_step": round(emitted / steps, 2),
+    tag = "mtp_verify_step_graphed_us" if graphed else "mtp_verify_step_us"
+    return {tag: round(t_total / steps * 1e6, 1), "mtp_tokens_per_step": round(emitted / steps, 2),
             "mtp_loop": f"{n_seq} sequences x (1 + 3 drafts), q4_0, ~{ctx} tokens each, prep + decode + accept/rollback, wall clock"}
 
 
