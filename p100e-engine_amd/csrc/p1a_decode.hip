@@ -141,22 +141,39 @@ __device__ __forceinline__ int sload_i32(const int32_t * p) {
     return *reinterpret_cast<const __attribute__((address_space(4))) int32_t *>(rfl64((size_t) p));
 }
 
-template <uint32_t KT, int D, int NT, int NWV, bool MULTI>
-__global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
+// SB ("single-buffered"): one K and one V slot per wave instead of two, so that two workgroups fit a CU's LDS (and register
+// file: 128 registers per lane) - for calls of many workgroups, where a second resident workgroup covers the start-up,
+// the fold and the memory round trips of the first. Tile t + 1 of K is then requested once the products with tile t of K
+// are done, V likewise; everything a lane computes, and the order it computes it in, is the same as in the double-buffered
+// kernel, so the partials are the same bits. One column tile of at most 8 live columns only (NT == 1, R <= 8).
+template <uint32_t KT, int D, int NT, int NWV, bool MULTI, bool SB>
+__global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
-    // four tile slots per wave (K and V, two each), plus a small per-wave table
-    __shared__ __attribute__((aligned(16))) char kb0[NWV * C::SLOT_B];
-    __shared__ __attribute__((aligned(16))) char vb0[NWV * C::SLOT_B];
-    __shared__ __attribute__((aligned(16))) char kv1[2 * NWV * C::SLOT_B];   // K slot 1, then V slot 1
-    char * const kb1 = kv1, * const vb1 = kv1 + NWV * C::SLOT_B;
-    static_assert(32 * D * 4 <= NWV * C::SLOT_B && 32 * C::QRS <= NWV * C::SLOT_B, "the Q copies (at most 32 columns) fit over the second K and V slots");
+    static_assert(!SB || NT == 1, "the single-buffered variant has one column tile");
+    // four tile slots per wave (K and V, two each), plus a small per-wave table. SB: one pool that holds one K slot, one
+    // V slot (and the q4_0 copy) per wave at the size of a tile, and is handed over to the fold as a whole afterwards:
+    // wave w parks 8 columns at a time, dim quarter k at PARK_B (4 w + k)
+    constexpr int SLB = SB ? C::TILE_B : C::SLOT_B;            // bytes per slot
+    constexpr int PARK_B = 8 * C::QDP * 4;                     // SB: one dim quarter of 8 parked columns
+    constexpr int POOL_T = NWV * (2 * C::TILE_B + C::VA_B), POOL_P = NWV * 4 * PARK_B;
+    __shared__ __attribute__((aligned(16))) char pool[SB ? (POOL_T > POOL_P ? POOL_T : POOL_P) : 16];
+    __shared__ __attribute__((aligned(16))) char kbA[SB ? 16 : NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char vbA[SB ? 16 : NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char kv1[SB ? 16 : 2 * NWV * C::SLOT_B];   // K slot 1, then V slot 1
+    __shared__ __attribute__((aligned(16))) char qown[SB ? 16 * C::QRS : 16];          // SB: the f16 Q table (first the fp32 copy of up to 8 rows)
+    char * const kb0 = SB ? pool : kbA, * const vb0 = SB ? pool + NWV * C::TILE_B : vbA;
+    char * const kb1 = SB ? kb0 : kv1, * const vb1 = SB ? vb0 : kv1 + NWV * C::SLOT_B;
+    static_assert(SB || (32 * D * 4 <= NWV * C::SLOT_B && 32 * C::QRS <= NWV * C::SLOT_B), "the Q copies (at most 32 columns) fit over the second K and V slots");
+    static_assert(!SB || 8 * D * 4 <= 16 * C::QRS, "SB: the fp32 copy of 8 rows fits where the f16 table of 16 goes");
     // q8_0 with two column tiles has no registers left for 64 dwords of Q operands (spills there cost more than their
     // traffic: the compiler can only wait for a reload with "no vector memory operation outstanding", tiles included):
     // that variant keeps the f16 Q table and reads its operands from it tile after tile
-    constexpr bool QLDS = KT == P1A_KV_Q8_0 && NT == 2;
-    __shared__ __attribute__((aligned(16))) char qtab[QLDS ? 32 * C::QRS : 16];
+    // (SB, 128 registers: likewise, whatever the type; its table has 8 columns and lanes c and c + 8 read the same one - the
+    // columns past the live ones are never weighted)
+    constexpr bool QLDS = (KT == P1A_KV_Q8_0 && NT == 2) || SB;
+    __shared__ __attribute__((aligned(16))) char qtab[QLDS && !SB ? 32 * C::QRS : 16];
     __shared__ __attribute__((aligned(16))) char tabs[NWV * C::TAB_B];
-    __shared__ __attribute__((aligned(16))) char vab[NWV * C::VA_B + 16];
+    __shared__ __attribute__((aligned(16))) char vab[SB ? 16 : NWV * C::VA_B + 16];
 
     const int lane = threadIdx.x & 63, wave = rfl(threadIdx.x >> 6);
     const int c = lane & 15, g = lane >> 4;
@@ -192,10 +209,10 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
     int pg0_early = 0;
     if (ptab) pg0_early = sload_i32(ptab + idx_early);
     const int p0v = P.pos_rows ? 0 : (P.p0_dev ? *P.p0_dev : P.p0);
-    char * const ks0 = kb0 + wave * C::SLOT_B, * const ks1 = kb1 + wave * C::SLOT_B;
-    char * const vs0 = vb0 + wave * C::SLOT_B, * const vs1 = vb1 + wave * C::SLOT_B;
+    char * const ks0 = kb0 + wave * SLB, * const ks1 = kb1 + wave * SLB;
+    char * const vs0 = vb0 + wave * SLB, * const vs1 = vb1 + wave * SLB;
     char * const tab = tabs + wave * C::TAB_B;
-    char * const va = vab + wave * C::VA_B;
+    char * const va = (SB ? pool + 2 * NWV * C::TILE_B : vab) + wave * C::VA_B;
 
     // column -> row of the group (at most 4 rows: three comparisons instead of a division)
     auto row_of = [&](int col) { return (col >= P.GQA) + (col >= 2 * P.GQA) + (col >= 3 * P.GQA); };
@@ -260,9 +277,10 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
         const int last = n_max - 1 - ts;
         const int i = rd * 64 + lane;
         uint32_t off = soff[rd];
-        if (last < 15) {
-            const int key = i / C::CPK, cir = i - key * C::CPK;
-            off = (uint32_t) (min(key, last) * rowb + (int) head_off + cir * 16);
+        if (last < 15) {   // (the last tile of a sequence only: worked out here, from scratch, rather than kept in registers)
+            int ii = i;
+            asm volatile("" : "+v"(ii));
+            off -= (uint32_t) (max(ii / C::CPK - last, 0) * rowb);
         }
         if (C::NCH % 64 == 0 || i < C::NCH) dma16(b0, off, lds_addr(slot) + rd * 1024);
     };
@@ -287,10 +305,34 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
     // This wave's share of the Q rows -> LDS (fp32, column col at col * 4 D bytes of K slot 1; lane i brings floats
     // 4 i .. 4 i + 3). These requests are OLDER than the tile requests that follow, so waiting for them below does not
     // wait for a tile.
+    // (SB with more than 8 live columns has no room for their fp32 copy: every thread fetches its pieces itself, scales and
+    // rounds them and writes them to the table - ahead of the tile requests, since the compiler's wait for such a load is a
+    // wait for everything outstanding)
+    const bool q_direct = SB && R > 8;
+    if (q_direct) {
+        constexpr int NPC = (16 * (D / 4) + NWV * 64 - 1) / (NWV * 64);
+        float4 a[NPC];
+#pragma unroll
+        for (int k = 0; k < NPC; ++k) {
+            const int i = threadIdx.x + k * NWV * 64, col = i / (D / 4), d4 = i - col * (D / 4);
+            a[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (col < R) {
+                const int t = row_of(col), hh = col - t * P.GQA;
+                a[k] = *reinterpret_cast<const float4 *>(P.q + ((size_t) (row0 + t) * P.Hq + (size_t) hk * P.GQA + hh) * D + 4 * d4);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < NPC; ++k) {
+            const int i = threadIdx.x + k * NWV * 64, col = i / (D / 4), d4 = i - col * (D / 4);
+            const float s = P.qscale;
+            if (col < 16) *reinterpret_cast<h4 *>(qown + col * C::QRS + d4 * 8) = h4{scale_to_half(a[k].x, s), scale_to_half(a[k].y, s), scale_to_half(a[k].z, s), scale_to_half(a[k].w, s)};
+        }
+    } else {
     for (int col = wave; col < R; col += NWV) {
         const int t = row_of(col), hh = col - t * P.GQA;
         const float * qr = P.q + ((size_t) (row0 + t) * P.Hq + (size_t) hk * P.GQA + hh) * D;
-        if (lane < D / 4) dma16(reinterpret_cast<const char *>(qr), lane * 16, lds_addr(kb1) + col * (D * 4));
+        if (lane < D / 4) dma16(reinterpret_cast<const char *>(qr), lane * 16, lds_addr(SB ? qown : kb1) + col * (D * 4));
+    }
     }
     request_k0(true);
     request_v0();
@@ -299,15 +341,27 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
     // piece - into an f16 table over V slot 1 (rows padded: conflict-free reads), and every lane picks its operands
     // out of that. (While a workgroup's requests queue up at the memory pipeline a wave cannot issue anything else:
     // what little work there is before the first tile is best kept short.)
-    if (tile_start(0) < n_max) wait_vm_imm<2 * C::NRND>(); else wait_vm_imm<0>();
+    if (!q_direct) { if (tile_start(0) < n_max) wait_vm_imm<2 * C::NRND>(); else wait_vm_imm<0>(); }
     __syncthreads();
-    char * const qt = QLDS ? qtab : vb1;
+    char * const qt = SB ? qown : QLDS ? qtab : vb1;
+    if constexpr (SB) {   // in place: at most one piece per thread (8 columns), read by all before any is written
+        static_assert(8 * (D / 4) <= NWV * 64, "SB: one piece of Q per thread");
+        if (!q_direct) {
+            const int i = threadIdx.x, col = i / (D / 4), d = 4 * (i - col * (D / 4));
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (col < R) a = *reinterpret_cast<const float4 *>(qown + (size_t) i * 16);
+            __syncthreads();
+            const float s = P.qscale;
+            if (col < 8) *reinterpret_cast<h4 *>(qt + col * C::QRS + d * 2) = h4{scale_to_half(a.x, s), scale_to_half(a.y, s), scale_to_half(a.z, s), scale_to_half(a.w, s)};
+        }
+    } else {
     for (int i = threadIdx.x; i < (QLDS ? 32 : R) * (D / 4); i += NWV * 64) {
         const int col = i / (D / 4), d = 4 * (i - col * (D / 4));
         float4 a = make_float4(0.f, 0.f, 0.f, 0.f);          // (columns past the live ones: zero operands)
         if (col < R) a = *reinterpret_cast<const float4 *>(kb1 + (size_t) i * 16);
         const float s = P.qscale;
         *reinterpret_cast<h4 *>(qt + col * C::QRS + d * 2) = h4{scale_to_half(a.x, s), scale_to_half(a.y, s), scale_to_half(a.z, s), scale_to_half(a.w, s)};
+    }
     }
     __syncthreads();
     h8 qf[QLDS ? 1 : NT][QLDS ? 1 : C::NMF];
@@ -327,7 +381,10 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
             qf[r][m] = livec ? h8{a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]} : h8{z, z, z, z, z, z, z, z};
         }
     }
-    __syncthreads();                                          // both copies are done with: tile 1 may be requested
+    if constexpr (!SB) __syncthreads();                       // both copies are done with: tile 1 may be requested
+    const char * qrow[NT];                                    // QLDS: this lane's row of the table, per column tile
+#pragma unroll
+    for (int r = 0; r < NT; ++r) qrow[r] = qt + (SB ? (R > 8 ? c : (c & 7)) : 16 * r + c) * C::QRS;
     f4 o[NT][C::NDT];
     f4 ol[NT];
     float m_run[NT];
@@ -370,8 +427,13 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
             for (int m = 0; m < C::NMF; ++m) {
                 const h8 a = *reinterpret_cast<const h8 *>(krow + (4 * m + g) * 16);
 #pragma unroll
-                for (int r = 0; r < NT; ++r) s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qf[r][m], s[r], 0, 0, 0);
-                if (have_n && m < C::NRND) fetch_round(ksn, kn, tn, m);
+                for (int r = 0; r < NT; ++r) {
+                    h8 qo;
+                    if constexpr (QLDS) qo = *reinterpret_cast<const h8 *>(qrow[r] + (32 * m + 8 * g) * 2);
+                    else qo = qf[r][m];
+                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qo, s[r], 0, 0, 0);
+                }
+                if (!SB && have_n && m < C::NRND) fetch_round(ksn, kn, tn, m);
             }
         } else if constexpr (KT == P1A_KV_Q4_0) {   // 8 blocks of 18 B: f16 scale, then 16 nibble bytes (2-byte aligned)
 #pragma unroll
@@ -389,8 +451,15 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
                 const u2 lo = deq4n(w & 0x0f0f0f0fu, dd), hi = deq4n((w >> 4) & 0x0f0f0f0fu, dd);
                 const u4 a = {lo.lo, lo.hi, hi.lo, hi.hi};
 #pragma unroll
-                for (int r = 0; r < NT; ++r) s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), qf[r][b], s[r], 0, 0, 0);
-                if (have_n && b < C::NRND) fetch_round(ksn, kn, tn, b);
+                for (int r = 0; r < NT; ++r) {
+                    h8 qo;
+                    if constexpr (QLDS) {
+                        const h4 x = *reinterpret_cast<const h4 *>(qrow[r] + (32 * b + 4 * g) * 2), y = *reinterpret_cast<const h4 *>(qrow[r] + (32 * b + 16 + 4 * g) * 2);
+                        qo = h8{x[0], x[1], x[2], x[3], y[0], y[1], y[2], y[3]};
+                    } else qo = qf[r][b];
+                    s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), qo, s[r], 0, 0, 0);
+                }
+                if (!SB && have_n && b < C::NRND) fetch_round(ksn, kn, tn, b);
             }
         } else {   // q8_0: 16 B of scales, then 16 chunks of 16 codes
             const i4 sc = *reinterpret_cast<const i4 *>(krow);
@@ -407,19 +476,24 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
                 for (int r = 0; r < NT; ++r) {
                     h8 q0, q1;
                     if constexpr (QLDS) {   // operands 2 jj and 2 jj + 1 of column 16 r + c: 16 consecutive halves of its table row
-                        const char * qr = qtab + (16 * r + c) * C::QRS + 32 * (4 * jj + g);
+                        const char * qr = qrow[r] + 32 * (4 * jj + g);
                         q0 = *reinterpret_cast<const h8 *>(qr);
                         q1 = *reinterpret_cast<const h8 *>(qr + 16);
                     } else { q0 = qf[r][2 * jj]; q1 = qf[r][2 * jj + 1]; }
                     s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a0), q0, s[r], 0, 0, 0);
                     s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a1), q1, s[r], 0, 0, 0);
                 }
-                if (have_n && jj < C::NRND) fetch_round(ksn, kn, tn, jj);
+                if (!SB && have_n && jj < C::NRND) fetch_round(ksn, kn, tn, jj);
             }
         }
-        if (have_n) {   // the rounds the product loop had no place for
+        if (!SB && have_n) {   // the rounds the product loop had no place for
 #pragma unroll
             for (int rd = (KT == P1A_KV_Q8_0 ? C::NMF / 2 : C::NMF); rd < C::NRND; ++rd) fetch_round(ksn, kn, tn, rd);
+        }
+        if (SB && have_n) {    // the K slot is free once its last fragment has been read
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ksn, kn, tn, rd);
         }
 
         // ---- online softmax (log2 domain); column = query row, this lane holds keys ts + 4 g + i ----
@@ -470,7 +544,7 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
                 const h4 a = __builtin_bit_cast(h4, w);
 #pragma unroll
                 for (int r = 0; r < NT; ++r) o[r][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[r], o[r][j], 0, 0, 0);
-                if (have_n && j < C::NRND) fetch_round(vsn, vn, tn, j);
+                if (!SB && have_n && j < C::NRND) fetch_round(vsn, vn, tn, j);
             }
         } else if constexpr (KT == P1A_KV_Q4_0) {
             {   // re-align: nibble bytes of block bb of a key -> va[key][bb][16] (8-byte aligned for the transposing read);
@@ -517,7 +591,7 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
                         o[r][2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a1), pb[r], o[r][2 * b + 1], 0, 0, 0);
                     }
                 }
-                if (have_n && p < C::NRND) fetch_round(vsn, vn, tn, p);
+                if (!SB && have_n && p < C::NRND) fetch_round(vsn, vn, tn, p);
             }
         } else {
             {   // transposed scale table tab[block][key] (f16, 32 B per block)
@@ -542,10 +616,15 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
                     o[r][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a0), pb[r], o[r][j], 0, 0, 0);
                     o[r][j + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a1), pb[r], o[r][j + 1], 0, 0, 0);
                 }
-                if (have_n && j / 2 < C::NRND) fetch_round(vsn, vn, tn, j / 2);
+                if (!SB && have_n && j / 2 < C::NRND) fetch_round(vsn, vn, tn, j / 2);
             }
         }
         static_assert(C::NRND <= (KT == P1A_KV_F16 ? C::NDT : KT == P1A_KV_Q8_0 ? C::NDT / 2 : C::NMF / 2), "the PV loop must have room for every V load");
+        if (SB && have_n) {    // the V slot likewise
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vsn, vn, tn, rd);
+        }
 #pragma unroll
         for (int r = 0; r < NT; ++r) ol[r] = __builtin_amdgcn_mfma_f32_16x16x16f16(ones, pb[r], ol[r], 0, 0, 0);
     };
@@ -556,30 +635,39 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
     }
     // ---- fold the waves of the workgroup (in wave order) and write one partial per (workgroup, head); the 16
     // columns of one MFMA tile at a time, so that a column is merged the same way whatever NT is. A wave parks its
-    // accumulators in its own (now idle) slots, dim quarter k in slot array k, and (m, l) in its table ----
+    // accumulators in its own (now idle) slots, dim quarter k in slot array k (SB: in its share of the pool, 8 columns at
+    // a time), and (m, l) in its table ----
     constexpr int QD = D / 4;                                 // dims per quarter
-    auto st = [&](int k) -> char * { return k == 0 ? kb0 : k == 1 ? kb1 : k == 2 ? vb0 : vb1; };
+    constexpr int PC = SB ? 8 : 16;                           // columns parked at a time
+    // (lane coordinates worked out afresh: what is derived from them here need not live in registers through the key loop)
+    int tid_f = threadIdx.x;
+    asm volatile("" : "+v"(tid_f));
+    const int c_f = tid_f & 15, g_f = (tid_f >> 4) & 3;
+    auto park = [&](int w, int k) -> float * {                // dim quarter k of wave w
+        if constexpr (SB) return reinterpret_cast<float *>(pool + (4 * w + k) * PARK_B);
+        else return reinterpret_cast<float *>((k == 0 ? kb0 : k == 1 ? kb1 : k == 2 ? vb0 : vb1) + w * C::SLOT_B);
+    };
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         const int Rr = min(16, R - 16 * r);                  // live columns of this tile
-        if (r) __syncthreads();
-        if (c < Rr) {
+        for (int h0 = 0; h0 < Rr; h0 += PC) {                // (one round unless SB)
+        const int he = min(h0 + PC, Rr);
+        if (r || h0 || SB) __syncthreads();                   // (SB: the pool changes hands once every wave is done with its tiles)
+        if (c_f >= h0 && c_f < he) {
 #pragma unroll
-            for (int j = 0; j < C::NDT; ++j) {
-                float * dst = reinterpret_cast<float *>(st(j / (C::NDT / 4)) + wave * C::SLOT_B);
-                *reinterpret_cast<f4 *>(dst + c * C::QDP + 16 * (j % (C::NDT / 4)) + 4 * g) = o[r][j];
-            }
-            if (g == 0) {
-                reinterpret_cast<float *>(tab)[c] = m_run[r];
-                reinterpret_cast<float *>(tab)[16 + c] = ol[r][0];
-            }
+            for (int j = 0; j < C::NDT; ++j)
+                *reinterpret_cast<f4 *>(park(wave, j / (C::NDT / 4)) + (c_f - h0) * C::QDP + 16 * (j % (C::NDT / 4)) + 4 * g_f) = o[r][j];
+        }
+        if (h0 == 0 && c_f < Rr && g_f == 0) {
+            reinterpret_cast<float *>(tab)[c_f] = m_run[r];
+            reinterpret_cast<float *>(tab)[16 + c_f] = ol[r][0];
         }
         __syncthreads();
-        // 32 lanes per column: the factors of a column (one per wave; a wave that saw no visible key parked zeros and
+        // LPC lanes per column: the factors of a column (one per wave; a wave that saw no visible key parked zeros and
         // gets the factor 0) are worked out once per lane and serve all the dims the lane folds
-        constexpr int LPC = 32;
-        for (int cc = threadIdx.x / LPC; cc < Rr; cc += NWV * 64 / LPC) {
-            const int dl = threadIdx.x % LPC;
+        constexpr int LPC = SB ? 64 : 32;
+        for (int cc = h0 + tid_f / LPC; cc < he; cc += NWV * 64 / LPC) {
+            const int dl = tid_f % LPC;
             float mw[NWV], lw[NWV], fw[NWV];
 #pragma unroll
             for (int w = 0; w < NWV; ++w) {
@@ -602,11 +690,9 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
 #pragma unroll
             for (int d4 = dl; d4 < D / 4; d4 += LPC) {
                 const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
-                const char * sbase = st(qtr);
                 f4 aw[NWV];
 #pragma unroll
-                for (int w = 0; w < NWV; ++w)
-                    aw[w] = *reinterpret_cast<const f4 *>(reinterpret_cast<const float *>(sbase + w * C::SLOT_B) + cc * C::QDP + dq);
+                for (int w = 0; w < NWV; ++w) aw[w] = *reinterpret_cast<const f4 *>(park(w, qtr) + (cc - h0) * C::QDP + dq);
                 f4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int w = 0; w < NWV; ++w) acc += aw[w] * fw[w];
@@ -620,6 +706,7 @@ __global__ void __launch_bounds__(NWV * 64, 1) dec_mfma_k(const dec_params P) {
                 pm[0] = M;
                 pm[1] = l;
             }
+        }
         }
     }
     }   // streams of this workgroup
@@ -878,15 +965,23 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     P.hkv_sh = -1;
     for (int sh = 0; sh < 16; ++sh) if ((1 << sh) == c.Hkv) P.hkv_sh = sh;
     P.npt = c.pt ? (int) (((long long) c.n_ctx + (1LL << c.psh) - 1) >> c.psh) : 0;
-    const dim3 grid(pl.nsplit / P.spw * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
     constexpr bool big_tiles = KT == P1A_KV_F16 && D == 256;
-#define P1A_DEC(NT_, NW_) do { if (P.spw > 1) dec_mfma_k<KT, D, NT_, NW_, true><<<grid, NW_ * 64, 0, s>>>(P); \
-                               else dec_mfma_k<KT, D, NT_, NW_, false><<<grid, NW_ * 64, 0, s>>>(P); } while (0)
+    // A call of at least two workgroups per CU whose row groups fit one column tile takes the single-buffered variant, two
+    // workgroups to a CU (same partials, bit for bit; measured at 24 / 4 heads, D = 256: 8 q8_0 slots of 1 K ... 27 K 56 ->
+    // 47 us, 4 x 64 K q4_0 single rows 92 -> 73 us, 16 x 2 rows q4_0 at 16 K 143 -> 115 us, 32 slots of 2 ... 5 K 104 -> 71 us).
+    // It walks one stream per workgroup: the second resident workgroup does what several streams per workgroup were for.
+    const long long wgs_all = (long long) pl.nsplit * c.Hkv * ((a.T + pl.RG - 1) / pl.RG);
+    const bool sb = !big_tiles && pl.NT == 1 && wgs_all >= 2LL * (a.cus > 0 ? a.cus : 256);
+    if (sb) P.spw = 1;
+    const dim3 grid(pl.nsplit / P.spw * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
+#define P1A_DEC(NT_, NW_) do { if (P.spw > 1) dec_mfma_k<KT, D, NT_, NW_, true, false><<<grid, NW_ * 64, 0, s>>>(P); \
+                               else dec_mfma_k<KT, D, NT_, NW_, false, false><<<grid, NW_ * 64, 0, s>>>(P); } while (0)
     if constexpr (big_tiles) {
         if (pl.NT == 1) P1A_DEC(1, 4);
         else P1A_DEC(2, 4);
     } else {
-        if (pl.NT == 1) P1A_DEC(1, 8);
+        if (sb) dec_mfma_k<KT, D, 1, 8, false, true><<<grid, 512, 0, s>>>(P);
+        else if (pl.NT == 1) P1A_DEC(1, 8);
         else P1A_DEC(2, 8);
     }
 #undef P1A_DEC

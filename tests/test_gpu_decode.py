@@ -201,6 +201,33 @@ def test_config4_verify_blocks(p1a, kv_type):
     check(out.cpu().numpy(), ref, "config 4 (reduced)")
 
 
+@pytest.mark.parametrize("kv_type,Hq,Hkv,D,rows", [(O.KV_Q8_0, 24, 4, 256, 1), (O.KV_Q8_0, 24, 4, 256, 2), (O.KV_Q4_0, 24, 4, 256, 1),
+                                                   (O.KV_Q4_0, 24, 4, 256, 2), (O.KV_F16, 32, 8, 128, 1), (O.KV_F16, 32, 8, 128, 2),
+                                                   (O.KV_F16, 16, 4, 64, 4), (O.KV_Q8_0, 32, 4, 256, 2)])
+def test_two_workgroups_per_cu_variant(p1a, kv_type, Hq, Hkv, D, rows):
+    """A call of two or more workgroups per CU with one column tile per row group runs a kernel variant with half the tile
+    slots (two workgroups share a CU): 5 sequences of unequal depth (one shorter than a unit, one a single key), 1 ... 4 rows
+    each, 6 ... 16 live columns - every row vs the oracle and bit for bit the row of a call of its own, which is small
+    enough to take the other variant."""
+    psh = 7
+    lens = [2300, 37, 1, 900, 4100][:5]
+    lens = [max(n, rows) for n in lens]
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, lens, seed=71)
+    T = len(lens) * rows
+    q, _, _, gate = I.qkv(72, 1, T, Hq, Hkv, D)
+    pos = np.array([n - rows + t for n in lens for t in range(rows)], np.int32)
+    rtab = np.array([s * pool.maxp for s in range(len(lens)) for _ in range(rows)], np.int32)
+    ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, 1 / 16, gate=gate)
+    out = torch.full((T, Hq, D), float("nan"), device="cuda")
+    p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, T, dev(pos), Hq, 1 / 16, gate=dev(gate), rows_per_seq=rows)
+    check(out.cpu().numpy(), ref, f"{len(lens)} sequences x {rows} rows, GQA {Hq // Hkv}, D {D}")
+    for t in range(T):
+        one = torch.empty((1, Hq, D), device="cuda")
+        p1a.attn_decode_rows(dev(q[t:t + 1]), pool.devkv.with_rows(dev(rtab[t:t + 1])), one, 1, dev(pos[t:t + 1]), Hq, 1 / 16,
+                             gate=dev(gate[t:t + 1]))
+        assert torch.equal(one[0], out[t]), t
+
+
 @pytest.mark.parametrize("kv_type,Hq,Hkv,rows", [(O.KV_Q8_0, 16, 2, 4), (O.KV_Q4_0, 32, 2, 2), (O.KV_F16, 16, 2, 4), (O.KV_Q8_0, 14, 2, 4)])
 def test_widest_row_groups(p1a, kv_type, Hq, Hkv, rows):
     """Row groups that fill both 16-column tiles (GQA 8 x 4 rows, GQA 16 x 2 rows: 32 live columns, the most the
