@@ -67,7 +67,6 @@ struct dec_params {
     int T, RG, Hq, Hkv, GQA;
     float qscale;     // softmax scale * log2(e)
     int nsplit;       // split streams
-    int spw;          // split streams one workgroup walks, one after the other (nsplit % spw == 0)
     int hkv_sh;       // log2(Hkv) when Hkv is a power of two, else -1
     int npt;          // page-table entries of one sequence (ceil(n_ctx / page positions)); 0 = contiguous
 };
@@ -147,7 +146,7 @@ __device__ __forceinline__ int sload_i32(const int32_t * p) {
 // the fold and the memory round trips of the first. Tile t + 1 of K is then requested once the products with tile t of K
 // are done, V likewise; everything a lane computes, and the order it computes it in, is the same as in the double-buffered
 // kernel, so the partials are the same bits. One column tile of at most 8 live columns only (NT == 1, R <= 8).
-template <uint32_t KT, int D, int NT, int NWV, bool MULTI, bool SB>
+template <uint32_t KT, int D, int NT, int NWV, bool SB>
 __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
     static_assert(!SB || NT == 1, "the single-buffered variant has one column tile");
@@ -158,12 +157,11 @@ __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_par
     constexpr int PARK_B = 8 * C::QDP * 4;                     // SB: one dim quarter of 8 parked columns
     constexpr int POOL_T = NWV * (2 * C::TILE_B + C::VA_B), POOL_P = NWV * 4 * PARK_B;
     __shared__ __attribute__((aligned(16))) char pool[SB ? (POOL_T > POOL_P ? POOL_T : POOL_P) : 16];
-    __shared__ __attribute__((aligned(16))) char kbA[SB ? 16 : NWV * C::SLOT_B];
-    __shared__ __attribute__((aligned(16))) char vbA[SB ? 16 : NWV * C::SLOT_B];
-    __shared__ __attribute__((aligned(16))) char kv1[SB ? 16 : 2 * NWV * C::SLOT_B];   // K slot 1, then V slot 1
+    // (one array, slot array k at k NWV SLOT_B: K slot 0, K slot 1, V slot 0, V slot 1 - the fold addresses them by number)
+    __shared__ __attribute__((aligned(16))) char slots[SB ? 16 : 4 * NWV * C::SLOT_B];
     __shared__ __attribute__((aligned(16))) char qown[SB ? 16 * C::QRS : 16];          // SB: the f16 Q table (first the fp32 copy of up to 8 rows)
-    char * const kb0 = SB ? pool : kbA, * const vb0 = SB ? pool + NWV * C::TILE_B : vbA;
-    char * const kb1 = SB ? kb0 : kv1, * const vb1 = SB ? vb0 : kv1 + NWV * C::SLOT_B;
+    char * const kb0 = SB ? pool : slots, * const vb0 = SB ? pool + NWV * C::TILE_B : slots + 2 * NWV * C::SLOT_B;
+    char * const kb1 = SB ? kb0 : slots + NWV * C::SLOT_B, * const vb1 = SB ? vb0 : slots + 3 * NWV * C::SLOT_B;
     static_assert(SB || (32 * D * 4 <= NWV * C::SLOT_B && 32 * C::QRS <= NWV * C::SLOT_B), "the Q copies (at most 32 columns) fit over the second K and V slots");
     static_assert(!SB || 8 * D * 4 <= 16 * C::QRS, "SB: the fp32 copy of 8 rows fits where the f16 table of 16 goes");
     // q8_0 with two column tiles has no registers left for 64 dwords of Q operands (spills there cost more than their
@@ -180,14 +178,9 @@ __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_par
     const int c = lane & 15, g = lane >> 4;
     // blockIdx.x -> (split stream, head group). Workgroups are dealt to the 8 XCDs round-robin by linear index, so
     // the kv heads of one split stream (which share cache lines) are given the same index mod 8.
-    // A workgroup may walk several split streams in turn (spw > 1, when a call has many more workgroups than the device
-    // has CUs): stream split, split + nsplit / spw, ... - every stream is computed and written exactly as if it had a
-    // workgroup of its own, only the per-workgroup set-up is shared.
     const int HG = P.Hkv;
-    const int spw = MULTI ? P.spw : 1;
-    const int nwgs = P.nsplit / spw;                          // workgroup-streams
     int split, hg;
-    if ((nwgs & 7) == 0) {
+    if ((P.nsplit & 7) == 0) {
         const int i = blockIdx.x, j = i >> 3;
         const int jq = P.hkv_sh >= 0 ? j >> P.hkv_sh : j / HG;
         hg = j - jq * HG;
@@ -243,11 +236,10 @@ __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_par
     // A workgroup none of whose streams holds a visible key (a short sequence in a batch: stream s is empty once s units
     // cover the sequence) writes the empty partials its streams would have ended with and is done.
     if (split * U >= n_max) {
-        for (int i = threadIdx.x; i < R * spw; i += NWV * 64) {
-            const int col = i % R, sw = i / R;
+        for (int col = threadIdx.x; col < R; col += NWV * 64) {
             const int t = row_of(col), hh = col - t * P.GQA;
             const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) hg * P.GQA + hh;
-            float * pm = P.part_ml + (row * P.nsplit + split + sw * nwgs) * 2;
+            float * pm = P.part_ml + (row * P.nsplit + split) * 2;
             pm[0] = NEG_INF;
             pm[1] = 0.f;
         }
@@ -390,13 +382,6 @@ __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_par
     f4 ol[NT];
     float m_run[NT];
     const h4 ones = {(half_t) 1, (half_t) 1, (half_t) 1, (half_t) 1};
-    for (int sw = 0; sw < spw; ++sw) {
-    if (MULTI && sw) {                                                 // the next stream: the slots are free behind this barrier
-        __syncthreads();
-        split += nwgs;
-        request_k0(false);
-        request_v0();
-    }
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         m_run[r] = NEG_INF;
@@ -646,7 +631,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_par
     const int c_f = tid_f & 15, g_f = (tid_f >> 4) & 3;
     auto park = [&](int w, int k) -> float * {                // dim quarter k of wave w
         if constexpr (SB) return reinterpret_cast<float *>(pool + (4 * w + k) * PARK_B);
-        else return reinterpret_cast<float *>((k == 0 ? kb0 : k == 1 ? kb1 : k == 2 ? vb0 : vb1) + w * C::SLOT_B);
+        else return reinterpret_cast<float *>(slots + (k * NWV + w) * C::SLOT_B);
     };
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
@@ -715,7 +700,6 @@ __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_par
         if (SB || he - h0 <= NWV) fold_round(std::integral_constant<int, 64>{}); else fold_round(std::integral_constant<int, 32>{});
         }
     }
-    }   // streams of this workgroup
 }
 
 // ---- generic path: any D % 32 == 0 (<= 512), any GQA, every type; one wave per (split stream, q head, row) ----
@@ -904,7 +888,6 @@ struct dec_plan {
     int GQA, NW, NT, RG;
     int nsplit;    // split streams
     int NS;        // partials per output row (what merge_k folds)
-    int spw;       // split streams per workgroup
 };
 
 bool mfma_ok(const p1a_kv & c, int GQA) {
@@ -948,17 +931,6 @@ void finish_plan(dec_plan & p) {
     if (p.mfma) p.NS = p.nsplit;
 }
 
-// how many split streams a workgroup walks: 1 until the call has more than four workgroups per CU slot; then as many
-// as bring it back there (a power of two that divides nsplit; measured: 8 slots of unequal depth 89 -> 80 us at 2,
-// 91 us at 4 - fewer, longer workgroups balance worse). The partials do not depend on it.
-int streams_per_wg(const dec_plan & p, int Hkv, int T, int cus) {
-    const long long wgs = (long long) p.nsplit * Hkv * ((T + p.RG - 1) / p.RG);
-    const int per_round = cus;
-    int spw = 1;
-    while (spw * 2 <= p.nsplit && p.nsplit % (spw * 2) == 0 && wgs / spw > 4LL * per_round) spw *= 2;
-    return spw;
-}
-
 template <uint32_t KT, int D>
 int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hipStream_t s) {
     dec_params P;
@@ -967,7 +939,6 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     P.p0 = a.p0; P.p0_dev = a.p0_dev; P.pos_rows = a.pos_rows;
     P.T = a.T; P.RG = pl.RG; P.Hq = a.Hq; P.Hkv = c.Hkv; P.GQA = pl.GQA;
     P.qscale = a.scale * 1.4426950408889634f; P.nsplit = pl.nsplit;
-    P.spw = streams_per_wg(pl, c.Hkv, a.T, a.cus > 0 ? a.cus : 256);
     P.hkv_sh = -1;
     for (int sh = 0; sh < 16; ++sh) if ((1 << sh) == c.Hkv) P.hkv_sh = sh;
     P.npt = c.pt ? (int) (((long long) c.n_ctx + (1LL << c.psh) - 1) >> c.psh) : 0;
@@ -975,18 +946,17 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     // A call of at least two workgroups per CU whose row groups fit one column tile takes the single-buffered variant, two
     // workgroups to a CU (same partials, bit for bit; measured at 24 / 4 heads, D = 256: 8 q8_0 slots of 1 K ... 27 K 56 ->
     // 47 us, 4 x 64 K q4_0 single rows 92 -> 73 us, 16 x 2 rows q4_0 at 16 K 143 -> 115 us, 32 slots of 2 ... 5 K 104 -> 71 us).
-    // It walks one stream per workgroup: the second resident workgroup does what several streams per workgroup were for.
+    // (A workgroup walks ONE split stream whatever the call: letting it walk several in turn - fewer, longer workgroups
+    // for calls of many - measured slower on every shape tried, e.g. 8 x 4 rows q4_0 at 8 K 72 -> 60 us with one.)
     const long long wgs_all = (long long) pl.nsplit * c.Hkv * ((a.T + pl.RG - 1) / pl.RG);
     const bool sb = !big_tiles && pl.NT == 1 && wgs_all >= 2LL * (a.cus > 0 ? a.cus : 256);
-    if (sb) P.spw = 1;
-    const dim3 grid(pl.nsplit / P.spw * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
-#define P1A_DEC(NT_, NW_) do { if (P.spw > 1) dec_mfma_k<KT, D, NT_, NW_, true, false><<<grid, NW_ * 64, 0, s>>>(P); \
-                               else dec_mfma_k<KT, D, NT_, NW_, false, false><<<grid, NW_ * 64, 0, s>>>(P); } while (0)
+    const dim3 grid(pl.nsplit * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
+#define P1A_DEC(NT_, NW_) dec_mfma_k<KT, D, NT_, NW_, false><<<grid, NW_ * 64, 0, s>>>(P)
     if constexpr (big_tiles) {
         if (pl.NT == 1) P1A_DEC(1, 4);
         else P1A_DEC(2, 4);
     } else {
-        if (sb) dec_mfma_k<KT, D, 1, 8, false, true><<<grid, 512, 0, s>>>(P);
+        if (sb) dec_mfma_k<KT, D, 1, 8, true><<<grid, 512, 0, s>>>(P);
         else if (pl.NT == 1) P1A_DEC(1, 8);
         else P1A_DEC(2, 8);
     }
