@@ -147,7 +147,7 @@ __device__ __forceinline__ int sload_i32(const int32_t * p) {
 // are done, V likewise; everything a lane computes, and the order it computes it in, is the same as in the double-buffered
 // kernel, so the partials are the same bits. One column tile of at most 8 live columns only (NT == 1, R <= 8).
 template <uint32_t KT, int D, int NT, int NWV, bool SB>
-__global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_params P) {
+__global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
     static_assert(!SB || NT == 1, "the single-buffered variant has one column tile");
     // four tile slots per wave (K and V, two each), plus a small per-wave table. SB: one pool that holds one K slot, one
@@ -337,15 +337,23 @@ __global__ void __launch_bounds__(NWV * 64, SB ? 4 : 1) dec_mfma_k(const dec_par
     if (!q_direct) { if (tile_start(0) < n_max) wait_vm_imm<2 * C::NRND>(); else wait_vm_imm<0>(); }
     __syncthreads();
     char * const qt = SB ? qown : QLDS ? qtab : vb1;
-    if constexpr (SB) {   // in place: at most one piece per thread (8 columns), read by all before any is written
-        static_assert(8 * (D / 4) <= NWV * 64, "SB: one piece of Q per thread");
+    if constexpr (SB) {   // in place (8 columns): every piece is read, by the thread that will write it, before any is written
         if (!q_direct) {
-            const int i = threadIdx.x, col = i / (D / 4), d = 4 * (i - col * (D / 4));
-            float4 a = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (col < R) a = *reinterpret_cast<const float4 *>(qown + (size_t) i * 16);
+            constexpr int NPQ = (8 * (D / 4) + NWV * 64 - 1) / (NWV * 64);
+            float4 a[NPQ];
+#pragma unroll
+            for (int k = 0; k < NPQ; ++k) {
+                const int i = threadIdx.x + k * NWV * 64, col = i / (D / 4);
+                a[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (col < R) a[k] = *reinterpret_cast<const float4 *>(qown + (size_t) i * 16);
+            }
             __syncthreads();
             const float s = P.qscale;
-            if (col < 8) *reinterpret_cast<h4 *>(qt + col * C::QRS + d * 2) = h4{scale_to_half(a.x, s), scale_to_half(a.y, s), scale_to_half(a.z, s), scale_to_half(a.w, s)};
+#pragma unroll
+            for (int k = 0; k < NPQ; ++k) {
+                const int i = threadIdx.x + k * NWV * 64, col = i / (D / 4), d = 4 * (i - col * (D / 4));
+                if (col < 8) *reinterpret_cast<h4 *>(qt + col * C::QRS + d * 2) = h4{scale_to_half(a[k].x, s), scale_to_half(a[k].y, s), scale_to_half(a[k].z, s), scale_to_half(a[k].w, s)};
+            }
         }
     } else {
     for (int i = threadIdx.x; i < (QLDS ? 32 : R) * (D / 4); i += NWV * 64) {
@@ -949,11 +957,12 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     // (A workgroup walks ONE split stream whatever the call: letting it walk several in turn - fewer, longer workgroups
     // for calls of many - measured slower on every shape tried, e.g. 8 x 4 rows q4_0 at 8 K 72 -> 60 us with one.)
     const long long wgs_all = (long long) pl.nsplit * c.Hkv * ((a.T + pl.RG - 1) / pl.RG);
-    const bool sb = !big_tiles && pl.NT == 1 && wgs_all >= 2LL * (a.cus > 0 ? a.cus : 256);
+    const bool sb = pl.NT == 1 && wgs_all >= 2LL * (a.cus > 0 ? a.cus : 256);
     const dim3 grid(pl.nsplit * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
 #define P1A_DEC(NT_, NW_) dec_mfma_k<KT, D, NT_, NW_, false><<<grid, NW_ * 64, 0, s>>>(P)
     if constexpr (big_tiles) {
-        if (pl.NT == 1) P1A_DEC(1, 4);
+        if (sb) dec_mfma_k<KT, D, 1, 4, true><<<grid, 256, 0, s>>>(P);
+        else if (pl.NT == 1) P1A_DEC(1, 4);
         else P1A_DEC(2, 4);
     } else {
         if (sb) dec_mfma_k<KT, D, 1, 8, true><<<grid, 512, 0, s>>>(P);

@@ -203,7 +203,8 @@ def test_config4_verify_blocks(p1a, kv_type):
 
 @pytest.mark.parametrize("kv_type,Hq,Hkv,D,rows", [(O.KV_Q8_0, 24, 4, 256, 1), (O.KV_Q8_0, 24, 4, 256, 2), (O.KV_Q4_0, 24, 4, 256, 1),
                                                    (O.KV_Q4_0, 24, 4, 256, 2), (O.KV_F16, 32, 8, 128, 1), (O.KV_F16, 32, 8, 128, 2),
-                                                   (O.KV_F16, 16, 4, 64, 4), (O.KV_Q8_0, 32, 4, 256, 2)])
+                                                   (O.KV_F16, 16, 4, 64, 4), (O.KV_Q8_0, 32, 4, 256, 2), (O.KV_F16, 24, 4, 256, 1),
+                                                   (O.KV_F16, 24, 4, 256, 2)])
 def test_two_workgroups_per_cu_variant(p1a, kv_type, Hq, Hkv, D, rows):
     """A call of two or more workgroups per CU with one column tile per row group runs a kernel variant with half the tile
     slots (two workgroups share a CU): 5 sequences of unequal depth (one shorter than a unit, one a single key), 1 ... 4 rows
