@@ -65,6 +65,19 @@ __device__ __forceinline__ float max_swap32(float m) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 0\n\tv_max_f32 %0, %0, %1" : "+v"(a), "+v"(b));
     return a;
 }
+// the maximum over all 64 lanes, in every lane: four steps inside a row of 16 lanes on the data-parallel-primitive path
+// (lane ^ 1, lane ^ 2, mirrored halves of 8, mirrored row - no LDS round trip), then the four rows by the two swaps
+template <int CTRL> __device__ __forceinline__ float max_dpp(float x) {
+    const int xi = __builtin_bit_cast(int, x);
+    return fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(xi, xi, CTRL, 0xf, 0xf, false)));
+}
+__device__ __forceinline__ float wave_max(float x) {
+    x = max_dpp<0xB1>(x);     // quad_perm [1, 0, 3, 2]
+    x = max_dpp<0x4E>(x);     // quad_perm [2, 3, 0, 1]
+    x = max_dpp<0x141>(x);    // row_half_mirror
+    x = max_dpp<0x140>(x);    // row_mirror
+    return max_swap32(max_swap16(x));
+}
 __device__ __forceinline__ void a16_quant8(const f4 v4, int l8, void * qbuf, int t, int g, int ng, int T, bool store) {
 #pragma clang fp contract(off)
     float v[4] = {v4[0], v4[1], v4[2], v4[3]};

@@ -838,8 +838,7 @@ __global__ void __launch_bounds__(256) merge_k(const float * __restrict__ part_o
     }
     M = pr.x;
     for (int s0 = 64; s0 < NS; s0 += 64) if (s0 + lane < NS) M = fmaxf(M, ml[2 * (s0 + lane)]);
-#pragma unroll
-    for (int w = 1; w < 64; w <<= 1) M = fmaxf(M, __shfl_xor(M, w));
+    M = wave_max(M);
     for (int s0 = 0; s0 < NS; s0 += 8 * CH) {
         if (s0) {
             pr = make_float2(NEG_INF, 0.f);
