@@ -270,10 +270,15 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
         const int last = n_max - 1 - ts;
         const int i = rd * 64 + lane;
         uint32_t off = soff[rd];
-        if (last < 15) {   // (the last tile of a sequence only: worked out here, from scratch, rather than kept in registers)
-            int ii = i;
-            asm volatile("" : "+v"(ii));
-            off -= (uint32_t) (max(ii / C::CPK - last, 0) * rowb);
+        if (last < 15) {   // (the last tile of a sequence only)
+            if constexpr (SB) {   // worked out from scratch rather than from values kept in registers through the key loop
+                int ii = i;
+                asm volatile("" : "+v"(ii));
+                off -= (uint32_t) (max(ii / C::CPK - last, 0) * rowb);
+            } else {
+                const int key = i / C::CPK, cir = i - key * C::CPK;
+                off = (uint32_t) (min(key, last) * rowb + (int) head_off + cir * 16);
+            }
         }
         if (C::NCH % 64 == 0 || i < C::NCH) dma16(b0, off, lds_addr(slot) + rd * 1024);
     };
@@ -660,7 +665,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
         // LPC lanes per column: the factors of a column (one per wave; a wave that saw no visible key parked zeros and
         // gets the factor 0) are worked out once per lane and serve all the dims the lane folds. 64 lanes when the columns of
         // the round are few enough for that to keep every thread busy (a single row of 6 heads: 384 threads fold one
-        // float4 each instead of 192 folding two - 1.1 us off the kernel at 32 K), else 32; the sums are the same either way
+        // float4 each instead of 192 folding two), else 32; the sums are the same either way
         auto fold_round = [&](auto lpc_tag) {
         constexpr int LPC = decltype(lpc_tag)::value;
         for (int cc = h0 + tid_f / LPC; cc < he; cc += NWV * 64 / LPC) {
