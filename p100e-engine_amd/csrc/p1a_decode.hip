@@ -435,17 +435,24 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                 if (!SB && have_n && m < C::NRND) fetch_round(ksn, kn, tn, m);
             }
         } else if constexpr (KT == P1A_KV_Q4_0) {   // 8 blocks of 18 B: f16 scale, then 16 nibble bytes (2-byte aligned)
+            // nibble bytes 4 g .. 4 g + 3 of block b sit at 18 b + 2 + 4 g: a whole dword in odd blocks, the upper and
+            // lower halves of two neighbouring dwords in even ones (head rows start 16-byte aligned). The reads of block
+            // b + 1 are asked for before block b is expanded, so that an LDS round trip hides behind the expansion.
+            struct kraw { uint32_t d16, w0, w1; };
+            auto kread = [&](int b) {
+                kraw r;
+                r.d16 = *reinterpret_cast<const uint16_t *>(krow + 18 * b);
+                if (b & 1) { r.w0 = *reinterpret_cast<const uint32_t *>(krow + 18 * b + 2 + 4 * g); r.w1 = 0; }   // (b is a constant once unrolled)
+                else { const uint32_t * pw = reinterpret_cast<const uint32_t *>(krow + 18 * b + 4 * g); r.w0 = pw[0]; r.w1 = pw[1]; }
+                return r;
+            };
+            kraw kcur = kread(0);
 #pragma unroll
             for (int b = 0; b < C::NMF; ++b) {
-                // nibble bytes 4 g .. 4 g + 3 of block b sit at 18 b + 2 + 4 g: a whole dword in odd blocks, the upper and
-                // lower halves of two neighbouring dwords in even ones (head rows start 16-byte aligned)
-                const uint32_t d16 = *reinterpret_cast<const uint16_t *>(krow + 18 * b);
-                uint32_t w;
-                if (b & 1) w = *reinterpret_cast<const uint32_t *>(krow + 18 * b + 2 + 4 * g);   // (b is a constant once unrolled)
-                else {
-                    const uint32_t * pw = reinterpret_cast<const uint32_t *>(krow + 18 * b + 4 * g);
-                    w = __builtin_amdgcn_alignbit(pw[1], pw[0], 16);
-                }
+                kraw knxt = kcur;
+                if (b + 1 < C::NMF) knxt = kread(b + 1);
+                const uint32_t d16 = kcur.d16;
+                const uint32_t w = (b & 1) ? kcur.w0 : __builtin_amdgcn_alignbit(kcur.w1, kcur.w0, 16);
                 const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
                 const u2 lo = deq4n(w & 0x0f0f0f0fu, dd), hi = deq4n((w >> 4) & 0x0f0f0f0fu, dd);
                 const u4 a = {lo.lo, lo.hi, hi.lo, hi.hi};
@@ -459,12 +466,15 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                     s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), qo, s[r], 0, 0, 0);
                 }
                 if (!SB && have_n && b < C::NRND) fetch_round(ksn, kn, tn, b);
+                kcur = knxt;
             }
         } else {   // q8_0: 16 B of scales, then 16 chunks of 16 codes
             const i4 sc = *reinterpret_cast<const i4 *>(krow);
+            i4 wcur = *reinterpret_cast<const i4 *>(krow + 16 + g * 16);
 #pragma unroll
             for (int jj = 0; jj < C::NMF / 2; ++jj) {
-                const i4 w = *reinterpret_cast<const i4 *>(krow + 16 + (4 * jj + g) * 16);
+                const i4 w = wcur;
+                if (jj + 1 < C::NMF / 2) wcur = *reinterpret_cast<const i4 *>(krow + 16 + (4 * (jj + 1) + g) * 16);
                 const uint32_t sw = (uint32_t) sc[jj];
                 const uint32_t d16 = (g & 2) ? (sw >> 16) : (sw & 0xffffu);
                 const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
@@ -573,13 +583,21 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
             // the same keys, block 2 p + 1. Low nibbles are dims 32 b + c, high nibbles dims 32 b + 16 + c.
             const int kk = c >> 1, jb = c & 1;
             const char * vrow = va + (4 * g + (kk & 3)) * 144 + 16 * (kk >> 2) + 8 * jb;
+            i2 wvc = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) vrow);
+            h4 dvc[2] = {*reinterpret_cast<const h4 *>(tab + g * 8), *reinterpret_cast<const h4 *>(tab + 32 + g * 8)};
 #pragma unroll
             for (int p = 0; p < C::NMF / 2; ++p) {
-                const i2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) (vrow + p * 32));
+                const i2 w = wvc;
+                const h4 dvp[2] = {dvc[0], dvc[1]};
+                if (p + 1 < C::NMF / 2) {
+                    wvc = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) (vrow + (p + 1) * 32));
+                    dvc[0] = *reinterpret_cast<const h4 *>(tab + (2 * p + 2) * 32 + g * 8);
+                    dvc[1] = *reinterpret_cast<const h4 *>(tab + (2 * p + 3) * 32 + g * 8);
+                }
 #pragma unroll
                 for (int x = 0; x < 2; ++x) {
                     const int b = 2 * p + x;
-                    const h4 dv = *reinterpret_cast<const h4 *>(tab + b * 32 + g * 8);
+                    const h4 dv = dvp[x];
                     const uint32_t wx = (uint32_t) w[x];
                     const u2 lo = deq4n2(wx & 0x0f0f0f0fu, h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
                     const u2 hi = deq4n2((wx >> 4) & 0x0f0f0f0fu, h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
@@ -603,10 +621,16 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
             // same keys at dims 16 (j + 1) ..
             const int kk = c >> 1, jb = c & 1;
             const char * vrow = vs + (4 * g + (kk & 3)) * C::HB + 16 + 16 * (kk >> 2) + 8 * jb;
+            i2 wvc = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) vrow);
+            h4 dvc = *reinterpret_cast<const h4 *>(tab + g * 8);
 #pragma unroll
             for (int j = 0; j < C::NDT; j += 2) {
-                const i2 w = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) (vrow + j * 16));
-                const h4 dv = *reinterpret_cast<const h4 *>(tab + (j >> 1) * 32 + g * 8);
+                const i2 w = wvc;
+                const h4 dv = dvc;
+                if (j + 2 < C::NDT) {
+                    wvc = __builtin_amdgcn_ds_read_tr8_b64_v2i32((i2 __attribute__((address_space(3))) *) (vrow + (j + 2) * 16));
+                    dvc = *reinterpret_cast<const h4 *>(tab + ((j + 2) >> 1) * 32 + g * 8);
+                }
                 const u2 x0 = deq4((uint32_t) w[0], h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
                 const u2 x1 = deq4((uint32_t) w[1], h2{dv[0], dv[1]}, h2{dv[2], dv[3]});
                 const i2 a0 = {(int) x0.lo, (int) x0.hi}, a1 = {(int) x1.lo, (int) x1.hi};
