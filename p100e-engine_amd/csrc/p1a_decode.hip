@@ -13,7 +13,8 @@
 //   consecutive lanes cover one q8_0 head row), written by the memory pipeline straight into a wave-private LDS slot
 //   that is the linear image of those rows - no staging registers, no workgroup barrier in the key loop. K and V have
 //   two slots each; the loads of tile t + 1 are issued between the products of tile t, and the in-order vector-memory
-//   counter tells which tile has landed. The Q rows are the same for all waves of a workgroup: they are requested
+//   counter tells which tile has landed. (A second build of the kernel, SB, has one slot each and half the registers, so
+//   that two workgroups share a CU: calls of many workgroups take it, see dec_mfma_k.) The Q rows are the same for all waves of a workgroup: they are requested
 //   first (older than every tile request), once, straight into LDS, and scaled and rounded into an f16 table that the
 //   lanes pick their MFMA operands from.
 // Arithmetic
@@ -145,7 +146,7 @@ __device__ __forceinline__ int sload_i32(const int32_t * p) {
 // file: 128 registers per lane) - for calls of many workgroups, where a second resident workgroup covers the start-up,
 // the fold and the memory round trips of the first. Tile t + 1 of K is then requested once the products with tile t of K
 // are done, V likewise; everything a lane computes, and the order it computes it in, is the same as in the double-buffered
-// kernel, so the partials are the same bits. One column tile of at most 8 live columns only (NT == 1, R <= 8).
+// kernel, so the partials are the same bits. One column tile only (NT == 1, at most 16 live columns).
 template <uint32_t KT, int D, int NT, int NWV, bool SB>
 __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
@@ -167,8 +168,8 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     // q8_0 with two column tiles has no registers left for 64 dwords of Q operands (spills there cost more than their
     // traffic: the compiler can only wait for a reload with "no vector memory operation outstanding", tiles included):
     // that variant keeps the f16 Q table and reads its operands from it tile after tile
-    // (SB, 128 registers: likewise, whatever the type; its table has 8 columns and lanes c and c + 8 read the same one - the
-    // columns past the live ones are never weighted)
+    // (SB, 128 registers: likewise, whatever the type; with at most 8 live columns its table has 8 and lanes c and c + 8
+    // read the same one - the columns past the live ones are never weighted)
     constexpr bool QLDS = (KT == P1A_KV_Q8_0 && NT == 2) || SB;
     __shared__ __attribute__((aligned(16))) char qtab[QLDS && !SB ? 32 * C::QRS : 16];
     __shared__ __attribute__((aligned(16))) char tabs[NWV * C::TAB_B];
