@@ -267,7 +267,21 @@ def batched_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
         p1a.warmup(32, Hq, Hkv, D)
         sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 8, pos, Hq, scale, gate=gate)] * reps, 2)
     bb = sum(lens) * 2 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
-    return {"batched_8slots_q8_0_us": round(sec * 1e6, 2), "batched_GBs": round(bb / sec / 1e9, 1), "batched_ctx": lens}
+    res = {"batched_8slots_q8_0_us": round(sec * 1e6, 2), "batched_GBs": round(bb / sec / 1e9, 1), "batched_ctx": lens}
+    del kv, cr
+    # the widest call the library takes: 32 slots, short contexts (2 K ... 5 K) - per-workgroup set-up is most of it
+    lens32 = [2048 + 100 * i for i in range(32)]
+    kv, ppseq = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, D, psh, max(lens32), 32, seed=24, lens=lens32)
+    pos = torch.tensor([n - 1 for n in lens32], dtype=torch.int32, device="cuda")
+    rt = torch.tensor([s * ppseq for s in range(32)], dtype=torch.int32, device="cuda")
+    q32 = torch.randn((32, Hq, D), generator=g, device="cuda")
+    out32 = torch.empty((32, Hq, D), device="cuda")
+    cr = kv.with_rows(rt)
+    with torch.cuda.stream(stream):
+        sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q32, cr, out32, 32, pos, Hq, scale)] * reps, 2)
+    bb = sum(lens32) * 2 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
+    res.update({"batched_32slots_2K_5K_q8_0_us": round(sec * 1e6, 2), "batched_32slots_GBs": round(bb / sec / 1e9, 1)})
+    return res
 
 
 def mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, n_seq=4, ctx=65000, steps=30, graphed=False):

@@ -230,3 +230,40 @@ def test_captured_key_split_prefill_is_refused_or_exact(p1a):
             s2.synchronize()
             assert torch.equal(out, eager), rep
 
+
+
+def test_batched_rows_in_a_graph(p1a):
+    """A batched call (8 rows of 4 sequences at their own positions - the two-workgroups-per-CU build of the kernel) captured
+    once and replayed while the sequences grow: every replay equals the eager call and, row by row, the call of that row alone"""
+    Hq, Hkv, D, psh = 24, 4, 256, 6
+    lens = [900, 450, 1300, 70]
+    pool = Pool(p1a, O.KV_Q4_0, Hq, Hkv, D, psh, lens, seed=52)
+    rows = [(s, 0) for s in range(4) for _ in range(2)]
+    q = dev(I.normal(I.rng(53), (8, Hq, D)))
+    gate = dev(I.normal(I.rng(54), (8, Hq * D)))
+    rt = dev(np.array([s * pool.maxp for s, _ in rows], np.int32))
+    cr = pool.devkv.with_rows(rt)
+    pos = dev(np.zeros(8, np.int32))
+    out_g = torch.empty((8, Hq, D), device="cuda")
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        p1a.warmup(8, Hq, Hkv, D)
+        pos.copy_(torch.tensor([10, 11] * 4, dtype=torch.int32))
+        s.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            p1a.attn_decode_rows(q, cr, out_g, 8, pos, Hq, 1 / 16, gate=gate, rows_per_seq=2)
+        for back in (40, 20, 0):
+            ph = np.array([lens[sq] - 2 - back + t for sq in range(4) for t in range(2)], np.int32)
+            pos.copy_(torch.from_numpy(ph))
+            g.replay()
+            s.synchronize()
+            eager = torch.empty_like(out_g)
+            p1a.attn_decode_rows(q, cr, eager, 8, pos, Hq, 1 / 16, gate=gate, rows_per_seq=2)
+            s.synchronize()
+            assert torch.equal(out_g, eager), back
+            for t in range(8):
+                one = torch.empty((1, Hq, D), device="cuda")
+                p1a.attn_decode_rows(q[t:t + 1], pool.devkv.with_rows(rt[t:t + 1]), one, 1, pos[t:t + 1], Hq, 1 / 16, gate=gate[t:t + 1])
+                s.synchronize()
+                assert torch.equal(one[0], out_g[t]), (back, t)
