@@ -221,6 +221,22 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     }
     n_max = rfl(n_max);
     p_min = rfl(p_min);
+    // A workgroup none of whose streams holds a visible key (a short sequence in a batch: stream s is empty once s units
+    // cover the sequence) is done before it asks for anything else - a wide call of short sequences launches several of
+    // these for every workgroup that has work. It leaves the empty partials its stream would have ended with, unless the
+    // rows carry their own positions: merge_k then knows from those which streams to skip and never reads them.
+    if (split * U >= n_max) {
+        if (!P.pos_rows) {
+            for (int col = threadIdx.x; col < R; col += NWV * 64) {
+                const int t = row_of(col), hh = col - t * P.GQA;
+                const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) hg * P.GQA + hh;
+                float * pm = P.part_ml + (row * P.nsplit + split) * 2;
+                pm[0] = NEG_INF;
+                pm[1] = 0.f;
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
         const int col = 16 * r + c;
@@ -234,18 +250,6 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     // "nothing outstanding", and placed after the requests such a wait would also wait for the tiles.
 #pragma unroll
     for (int r = 0; r < NT; ++r) asm volatile("" : "+v"(plim[r]));
-    // A workgroup none of whose streams holds a visible key (a short sequence in a batch: stream s is empty once s units
-    // cover the sequence) writes the empty partials its streams would have ended with and is done.
-    if (split * U >= n_max) {
-        for (int col = threadIdx.x; col < R; col += NWV * 64) {
-            const int t = row_of(col), hh = col - t * P.GQA;
-            const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) hg * P.GQA + hh;
-            float * pm = P.part_ml + (row * P.nsplit + split) * 2;
-            pm[0] = NEG_INF;
-            pm[1] = 0.f;
-        }
-        return;
-    }
     const size_t head_off = (size_t) hk * C::HB;
     const int rowb = (int) P.pg.rowb;
 
