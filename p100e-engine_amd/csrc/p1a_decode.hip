@@ -197,7 +197,12 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     const int R = nr * P.GQA;                                 // live MFMA columns
     // the page-table entry of this wave's first tile is asked for before anything else (it is the first link of the
     // chain entry -> tile address -> tile); the index is clamped into the table, the entry is only used if the tile exists
-    const int32_t * ptab = kv_tab(P.pg, P.pos_rows ? row0 : 0);
+    // (the group's first position and its page-table row hang on the kernel arguments only: both scalar loads are issued
+    // before either value is used - one round trip for the two)
+    const bool has_rt = P.pg.pt && P.pg.rtab;
+    const int rt0 = has_rt ? sload_i32(P.pg.rtab + (P.pos_rows ? row0 : 0)) : 0;
+    const int pos_first = P.pos_rows ? sload_i32(P.pos_rows + row0) : 0;
+    const int32_t * ptab = P.pg.pt ? P.pg.pt + rt0 : nullptr;
     // (n_ctx only bounds the read here: an entry fetched through a clamped index is fetched again, unclamped, once the
     // tile is known to exist)
     const int idx_early = max(0, min((split * U + sub * 32) >> P.pg.psh, P.npt - 1));
@@ -215,7 +220,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     int plim[NT];
     int n_max = 0, p_min = 0x7fffffff;
     for (int t = 0; t < nr; ++t) {
-        const int pt_ = P.pos_rows ? P.pos_rows[row0 + t] : p0v + row0 + t;
+        const int pt_ = P.pos_rows ? (t ? P.pos_rows[row0 + t] : pos_first) : p0v + row0 + t;
         n_max = max(n_max, pt_ + 1);
         p_min = min(p_min, pt_);
     }
