@@ -704,6 +704,19 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
         constexpr int LPC = decltype(lpc_tag)::value;
         for (int cc = h0 + tid_f / LPC; cc < he; cc += NWV * 64 / LPC) {
             const int dl = tid_f % LPC;
+            // the parked accumulators are asked for first: they do not depend on the factors, whose table reads and
+            // exponentials then run under their LDS round trip instead of in front of it
+            constexpr int NIT = (D / 4 + LPC - 1) / LPC;
+            f4 aw[NIT][NWV];
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int d4 = dl + it * LPC;
+                if (D / 4 % LPC == 0 || d4 < D / 4) {
+                    const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
+#pragma unroll
+                    for (int w = 0; w < NWV; ++w) aw[it][w] = *reinterpret_cast<const f4 *>(park(w, qtr) + (cc - h0) * C::QDP + dq);
+                }
+            }
             float mw[NWV], lw[NWV], fw[NWV];
 #pragma unroll
             for (int w = 0; w < NWV; ++w) {
@@ -724,18 +737,17 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
             const int t = row_of(col), hh = col - t * P.GQA;
             const size_t row = (size_t) (row0 + t) * P.Hq + (size_t) hg * P.GQA + hh;
 #pragma unroll
-            for (int d4 = dl; d4 < D / 4; d4 += LPC) {
-                const int qtr = (4 * d4) / QD, dq = 4 * d4 - qtr * QD;
-                f4 aw[NWV];
+            for (int it = 0; it < NIT; ++it) {
+                const int d4 = dl + it * LPC;
+                if (D / 4 % LPC == 0 || d4 < D / 4) {
+                    f4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int w = 0; w < NWV; ++w) aw[w] = *reinterpret_cast<const f4 *>(park(w, qtr) + (cc - h0) * C::QDP + dq);
-                f4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int w = 0; w < NWV; ++w) acc += aw[w] * fw[w];
-                // (two column tiles = several rows per group: the partials are tens of megabytes and nothing here reads
-                // them again, so they go past the cache - measured -3 ... -5 % on 4-row verify calls, +6 % on a single row)
-                f4 * const po = reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4);
-                if (M != NEG_INF) { if constexpr (NT == 2) __builtin_nontemporal_store(acc, po); else *po = acc; }
+                    for (int w = 0; w < NWV; ++w) acc += aw[it][w] * fw[w];
+                    // (two column tiles = several rows per group: the partials are tens of megabytes and nothing here reads
+                    // them again, so they go past the cache - measured -3 ... -5 % on 4-row verify calls, +6 % on a single row)
+                    f4 * const po = reinterpret_cast<f4 *>(P.part_o + (row * P.nsplit + split) * D + 4 * d4);
+                    if (M != NEG_INF) { if constexpr (NT == 2) __builtin_nontemporal_store(acc, po); else *po = acc; }
+                }
             }
             if (dl == 0) {
                 float * pm = P.part_ml + (row * P.nsplit + split) * 2;
