@@ -151,7 +151,7 @@ int p1a_attn_decode_a16(const float *q, const p1a_kv *c, float *out, const float
  * same result bits, but the split partials live in a fixed array in device memory (P1A_NOALLOC_SCRATCH_BYTES, one copy per
  * GPU, held until the process ends) instead of the library's per-stream buffers, and the call never allocates or frees
  * anything. A call whose partials do not fit (T * Hq * splits * (D + 2) * 4 bytes; 8 rows of the 24 / 4 / 256 shape fit for
- * every KV type: 64 split streams for q8_0 / q4_0, 128 for f16) is refused with P1A_E_SCRATCH. Every call on one GPU shares that GPU's array: calls that overlap on one GPU
+ * every KV type: CUs / Hkv = 64 split streams on a 256-CU part) is refused with P1A_E_SCRATCH. Every call on one GPU shares that GPU's array: calls that overlap on one GPU
  * (two streams, two threads) race - serialise them. The array's address is looked up on the first call per device (or by
  * p1a_warmup).
  */
@@ -218,8 +218,24 @@ int p1a_warmup(int rows, int Hq, int Hkv, int D, void *stream);
  * attn_dec2_nsplit / attn_dec2_set_nsplit, src/fast/attn_dec2.cuh:19-20. Never change it between graph captures. */
 int p1a_get_nsplit(int Hkv);
 void p1a_set_nsplit(int n);
+/* Bytes of split scratch one decode call of these arguments needs (accumulators rounded up to 256 bytes, then the (m, l)
+ * pairs), and the bytes the library keeps per (device, stream) for a head shape - the larger of the two is what a first call
+ * allocates. A cache the MFMA kernel cannot take (misaligned base or page stride, pages of fewer than 16 positions, quantized
+ * types at D != 256) takes the generic kernel, which leaves more partials per row; both are covered. No GPU call is made
+ * (without a device the plan of a 256-CU part is returned). No counterpart in the reference, whose scratch size is a
+ * compile-time constant (src/fast/attn_dec2.cu:452-464). */
+size_t p1a_decode_scratch_bytes(const p1a_kv *c, int Hq, int T, int rows_per_seq);
+size_t p1a_decode_footprint_bytes(int Hq, int Hkv, int D);
+/* An identity of everything in this library that can change output BITS for a head shape on the current device: library
+ * version and numerics revision, CU count, split-stream count (P1A_DEC_SPLIT / p1a_set_nsplit included). Two processes with
+ * equal ids produce bit-identical attention outputs for equal inputs; the engine folds such switches into the numerics
+ * hash of its session files (src/tp_model.cu:3697-3735). The prefill key-split plan is a function of (T, p0, Hq) and the
+ * CU count, so it is covered. */
+#define P1A_NUMERICS_REV 3
+uint64_t p1a_numerics_id(int Hq, int Hkv);
 /* Re-read the environment switch that is baked into captured graphs (P1A_DEC_SPLIT, the split-stream count); returns 1
- * when it changed since it was last read (the caller must then drop its captured graphs), else 0.
+ * when it differs from what was last read - the very first read included, as in the reference - (the caller must then drop
+ * its captured graphs), else 0.
  * Replaces attn_dec2_reload_env, src/fast/attn_dec2.cuh:21 (called from src/tp_model.cu:3229). */
 int p1a_reload_env(void);
 /* Benchmarks only (no counterpart in the reference, whose benches time both kernels together): p1a_attn_decode without

@@ -9,7 +9,7 @@ KV_F16, KV_Q4_0, KV_Q8_0 = 1, 2, 8
 EXPORTS = [
     "p1a_kv_row_bytes", "p1a_kv_append", "p1a_kv_fill_random", "p1a_attn_prep", "p1a_attn_prep_mrope", "p1a_attn_decode", "p1a_attn_decode_a16", "p1a_attn_decode_noalloc", "p1a_a16_bytes", "p1a_ew_quant", "p1a_attn_prefill", "p1a_attn_prefill_scratch_bytes", "p1a_attn_prefill_key_splits",
     "p1a_sigmoid_mul", "p1a_warmup", "p1a_get_nsplit", "p1a_set_nsplit", "p1a_reload_env", "p1a_warmup_prefill", "p1a_set_prefill_staging_limit", "p1a_bench_decode_split_only", "p1a_bench_stream_read", "p1a_release", "p1a_last_error",
-    "p1a_version",
+    "p1a_version", "p1a_decode_scratch_bytes", "p1a_decode_footprint_bytes", "p1a_numerics_id",
     # include/p1a_pool.h
     "p1a_pool_create", "p1a_pool_destroy", "p1a_pool_n_pages", "p1a_pool_free_pages", "p1a_pool_max_pages", "p1a_pool_page_bytes",
     "p1a_pool_host_used", "p1a_pool_kv_seq", "p1a_pool_kv_rows", "p1a_pool_set_rows", "p1a_pool_state", "p1a_seq_create", "p1a_seq_free",
@@ -91,6 +91,12 @@ def lib():
     L.p1a_warmup.argtypes = [i32, i32, i32, i32, vp]
     L.p1a_get_nsplit.restype = i32
     L.p1a_get_nsplit.argtypes = [i32]
+    L.p1a_decode_scratch_bytes.restype = sz
+    L.p1a_decode_scratch_bytes.argtypes = [kvp, i32, i32, i32]
+    L.p1a_decode_footprint_bytes.restype = sz
+    L.p1a_decode_footprint_bytes.argtypes = [i32, i32, i32]
+    L.p1a_numerics_id.restype = ctypes.c_uint64
+    L.p1a_numerics_id.argtypes = [i32, i32]
     L.p1a_set_nsplit.restype = None
     L.p1a_set_nsplit.argtypes = [i32]
     L.p1a_reload_env.restype = i32
@@ -324,6 +330,18 @@ def get_nsplit(Hkv):
 
 def set_nsplit(n):
     lib().p1a_set_nsplit(n)
+
+
+def decode_scratch_bytes(c, Hq, T, rows_per_seq=1):
+    return int(lib().p1a_decode_scratch_bytes(ctypes.byref(c), Hq, T, rows_per_seq))
+
+
+def decode_footprint_bytes(Hq, Hkv, D):
+    return int(lib().p1a_decode_footprint_bytes(Hq, Hkv, D))
+
+
+def numerics_id(Hq, Hkv):
+    return int(lib().p1a_numerics_id(Hq, Hkv))
 
 
 def reload_env():

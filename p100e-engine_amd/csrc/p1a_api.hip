@@ -142,17 +142,21 @@ int nsplit_req() {
 void decode_footprint(int Hq, int Hkv, int D, size_t & need_o, size_t & need_ml) {
     p1a_kv c;
     memset(&c, 0, sizeof c);
-    c.Hkv = Hkv; c.D = D; c.k = c.v = (void *) 16;
+    c.Hkv = Hkv; c.D = D;
     need_o = need_ml = 0;
     const uint32_t types[3] = {P1A_KV_F16, P1A_KV_Q8_0, P1A_KV_Q4_0};
-    for (uint32_t ty : types)
-        for (int rg = 1; rg <= 4; ++rg) {
-            size_t o, m;
-            c.type = ty;
-            decode_scratch_need(c, Hq, P1A_MAX_ROWS, rg, nsplit_req(), cu_count(), o, m);
-            if (o > need_o) need_o = o;
-            if (m > need_ml) need_ml = m;
-        }
+    // (a cache the MFMA kernel cannot take - a misaligned base, short pages - goes to the generic kernel, which leaves more
+    // partials per row: both plans count, so that a warm-up also covers such caches)
+    for (uintptr_t base : {(uintptr_t) 16, (uintptr_t) 8})
+        for (uint32_t ty : types)
+            for (int rg = 1; rg <= 4; ++rg) {
+                size_t o, m;
+                c.type = ty;
+                c.k = c.v = (void *) base;
+                decode_scratch_need(c, Hq, P1A_MAX_ROWS, rg, nsplit_req(), cu_count(), o, m);
+                if (o > need_o) need_o = o;
+                if (m > need_ml) need_ml = m;
+            }
 }
 
 // ext / ext_bytes: split scratch brought by the caller of this function (the allocation-free entry point); nullptr = the
@@ -189,12 +193,19 @@ int decode_call(const float * q, const p1a_kv * c, float * out, const float * ga
         }
         a.part_o = reinterpret_cast<float *>(ext);
         a.part_ml = reinterpret_cast<float *>(reinterpret_cast<char *>(ext) + need_o);
+        a.cap_o = need_o; a.cap_ml = ext_bytes - need_o;
         return launch_decode(*c, a, s);
     }
+    // the footprint of the head shape (so that the pointer never changes again), and never less than THIS call needs
+    size_t real_o, real_ml;
+    decode_scratch_need(*c, Hq, T, a.rows_per_group, a.nsplit, a.cus, real_o, real_ml);
     decode_footprint(Hq, c->Hkv, c->D, need_o, need_ml);
+    if (real_o > need_o) need_o = real_o;
+    if (real_ml > need_ml) need_ml = real_ml;
     bufpair * sc = scratch_for(s, BUF_DECODE, need_o, need_ml);
     if (!sc) return P1A_E_SCRATCH;
     a.part_o = sc->o; a.part_ml = sc->ml;
+    a.cap_o = sc->cap_o; a.cap_ml = sc->cap_ml;
     return launch_decode(*c, a, s);
 }
 
@@ -390,9 +401,39 @@ int p1a_get_nsplit(int Hkv) {
 
 void p1a_set_nsplit(int n) { g_nsplit_override = n > 0 ? n : 0; }
 
+size_t p1a_decode_scratch_bytes(const p1a_kv * c, int Hq, int T, int rows_per_seq) {
+    if (!c || c->Hkv < 1 || Hq < c->Hkv || Hq % c->Hkv || T < 1) return 0;
+    int rg = decode_rows_per_group(*c, Hq, rows_per_seq < 1 ? 1 : rows_per_seq);
+    while (rows_per_seq > 1 && rows_per_seq % rg) --rg;
+    size_t o, m;
+    decode_scratch_need(*c, Hq, T, rg, nsplit_req(), cu_count(), o, m);
+    return ((o + 255) & ~(size_t) 255) + m;
+}
+
+size_t p1a_decode_footprint_bytes(int Hq, int Hkv, int D) {
+    if (Hkv < 1 || Hq < Hkv || Hq % Hkv || D < 32) return 0;
+    size_t o, m;
+    decode_footprint(Hq, Hkv, D, o, m);
+    return ((o + 255) & ~(size_t) 255) + m;
+}
+
+uint64_t p1a_numerics_id(int Hq, int Hkv) {
+    // FNV-1a over what fixes the summation order of the results on this device
+    uint64_t h = 1469598103934665603ull;
+    auto mix = [&](uint64_t v) { for (int i = 0; i < 8; ++i) { h ^= (v >> (8 * i)) & 0xff; h *= 1099511628211ull; } };
+    for (const char * p = p1a_version(); *p; ++p) { h ^= (unsigned char) *p; h *= 1099511628211ull; }
+    mix((uint64_t) P1A_NUMERICS_REV);
+    mix((uint64_t) cu_count());
+    mix((uint64_t) p1a_get_nsplit(Hkv < 1 ? 1 : Hkv));
+    mix((uint64_t) (Hq > 0 ? Hq : 0));
+    mix((uint64_t) (Hkv > 0 ? Hkv : 0));
+    return h;
+}
+
 int p1a_reload_env(void) {
     const int v = read_env_split();
-    const bool changed = g_env_split >= 0 && v != g_env_split;
+    // (the first read counts as a change, as in the reference, whose switch starts out unread: src/fast/attn_dec2.cu reload)
+    const bool changed = v != g_env_split;
     g_env_split = v;
     return changed ? 1 : 0;
 }

@@ -124,6 +124,7 @@ struct decode_args {
     bool skip_merge;      // benchmarks only: stop after the split-K kernel
     float * part_o;       // [T*Hq][nsplit][D]
     float * part_ml;      // [T*Hq][nsplit][2]
+    size_t cap_o, cap_ml; // bytes behind part_o / part_ml (a launch that would write past them is refused)
     void * qbuf;          // optional: a16 activation buffer of the (gated) output, [T][Hq*D] values
 };
 int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s);

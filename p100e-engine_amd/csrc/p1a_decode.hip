@@ -864,7 +864,9 @@ __global__ void __launch_bounds__(256) merge_k(const float * __restrict__ part_o
     const size_t row = blockIdx.x;
     const int NS_row = NS_all;                                // (the row stride of the partials)
     int NS = NS_all;
-    if (pos_rows && U > 0) NS = min(NS_all, pos_rows[row / Hq] / U + 1);
+    // (a row at a negative position - an idle slot - sees no key: no stream is read, and 0 / 0 gives the NaN row the
+    // reference's combine gives for n = 0)
+    if (pos_rows && U > 0) { const int pr_ = pos_rows[row / Hq]; NS = pr_ < 0 ? 0 : min(NS_all, pr_ / U + 1); }
     const int tid = threadIdx.x, lane = tid & 63, qd = tid & 31, sl = tid >> 5;
     const int d = blockIdx.y * MRG_DIMS + qd * 4;
     const bool live = d < D;
@@ -1044,6 +1046,12 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
     dec_plan pl = make_plan(c, a.Hq, a.rows_per_group, a.nsplit, a.cus);
     pl.RG = a.rows_per_group;
     finish_plan(pl);
+    // the partials of this launch: [T * Hq][NS][D] accumulators and [T * Hq][NS][2] (m, l) pairs
+    const size_t need_o = (size_t) a.T * a.Hq * pl.NS * c.D * sizeof(float), need_ml = (size_t) a.T * a.Hq * pl.NS * 2 * sizeof(float);
+    if (need_o > a.cap_o || need_ml > a.cap_ml) {
+        set_error("p1a_attn_decode: split partials of %zu + %zu bytes do not fit the scratch of %zu + %zu", need_o, need_ml, a.cap_o, a.cap_ml);
+        return P1A_E_SCRATCH;
+    }
     int rc;
     if (pl.mfma) {
         if (c.type == P1A_KV_Q8_0) rc = launch_mfma<P1A_KV_Q8_0, 256>(c, a, pl, s);

@@ -65,12 +65,13 @@ class Pool:
         return self.p1a.KVCache(self.type, self.lens[s], self.Hkv, self.D, dk.data_ptr(), dv.data_ptr(), keep=(dk, dv))
 
 
-def check(out, ref, what="", rel_l2_tol=None):
+def check(out, ref, what="", rel_l2_tol=None, flat=False):
     """max-abs <= 2e-3 (times max|ref| where the reference exceeds 1: the products run on f16 operands, whose error is
     relative - the criterion of the engine's own tests, tests/fast_attn_test.cu:75,217,269 - and outputs above 1 only
-    occur for contexts of a few keys) and rel-L2 <= 1e-3"""
+    occur for contexts of a few keys) and rel-L2 <= 1e-3. flat=True holds the max-abs to the plain 2e-3 whatever the
+    reference's magnitude: the benchmark configurations are stated that way."""
     ma, rl = I.errors(out, ref)
-    tol = I.MAX_ABS_TOL * max(1.0, float(np.max(np.abs(ref))))
+    tol = I.MAX_ABS_TOL * (1.0 if flat else max(1.0, float(np.max(np.abs(ref)))))
     rtol = I.REL_L2_TOL if rel_l2_tol is None else rel_l2_tol     # (only tests that craft scores far outside the model's range pass one)
     assert np.all(np.isfinite(out)), what
     flat = "flat 2e-3 bound held" if ma <= I.MAX_ABS_TOL else f"flat 2e-3 bound NOT held (max|ref|={float(np.max(np.abs(ref))):.3g})"

@@ -77,3 +77,40 @@ def test_reload_env(p1a):
         if old is not None:
             os.environ["P1A_DEC_SPLIT"] = old
         p1a.reload_env()
+
+
+def test_decode_scratch_need_never_exceeds_footprint(p1a):
+    """The per-(device, stream) buffers are sized once, at the footprint of a head shape. Whatever cache a later call of
+    that head shape brings - short pages, a misaligned base or page stride (the generic kernel: more partials per row),
+    any row grouping - its partials must fit that footprint. Host arithmetic only."""
+    from importlib import import_module
+    b = import_module("p100e-engine_amd.binding")
+    worst = 0
+    for Hq, Hkv, D in ((24, 4, 256), (4, 4, 256), (16, 2, 128), (8, 8, 64), (32, 2, 256), (4, 1, 64)):
+        fp = p1a.decode_footprint_bytes(Hq, Hkv, D)
+        assert fp > 0
+        for ty in (p1a.KV_F16, p1a.KV_Q8_0, p1a.KV_Q4_0):
+            for psh in range(0, 9):
+                for base, pstride_extra in ((4096, 0), (4096 + 8, 0), (4096, 8), (4096 + 2, 2)):
+                    for T, rps in ((1, 1), (9, 1), (32, 1), (32, 4), (12, 3), (16, 2)):
+                        kv = b.p1a_kv()
+                        kv.type, kv.Hkv, kv.D, kv.n_ctx = ty, Hkv, D, 1 << 14
+                        kv.k = kv.v = base
+                        kv.pt = 4096
+                        kv.psh = psh
+                        kv.pstride = (p1a.kv_row_bytes(ty, Hkv, D) << psh) + pstride_extra
+                        need = p1a.decode_scratch_bytes(kv, Hq, T, rps)
+                        assert 0 < need <= fp, (Hq, Hkv, D, ty, psh, base, T, rps, need, fp)
+                        worst = max(worst, need / fp)
+    assert worst > 0.5          # the footprint is not wildly oversized either
+
+
+def test_numerics_id_follows_the_split_count(p1a):
+    a = p1a.numerics_id(24, 4)
+    assert a == p1a.numerics_id(24, 4) and a != 0
+    try:
+        p1a.set_nsplit(24)
+        assert p1a.numerics_id(24, 4) != a
+    finally:
+        p1a.set_nsplit(0)
+    assert p1a.numerics_id(24, 4) == a

@@ -28,7 +28,7 @@ def test_config1_tiny_f16(p1a):
     q, _, _, _ = I.qkv(0, n, 1, Hq, Hkv, D, f16_inputs=True)
     ref = O.attn_rows(pool.host_seq(0), q, np.array([n - 1]), Hq, 0.125)
     out = run_decode(p1a, pool.dev_seq(0), q, 1, n - 1, Hq, 0.125)
-    check(out, ref, "config 1")
+    check(out, ref, "config 1", flat=True)
 
 
 @pytest.mark.parametrize("kv_type", TYPES)

@@ -35,7 +35,7 @@ def test_config2_decode_32k_q8_0(p1a):
     ref = O.attn_rows(pool.host_seq(0), q, np.array([n - 1], np.int32), Hq, 1 / 16, gate=gate)
     out = torch.empty((1, Hq, D), device="cuda")
     p1a.attn_decode(dev(q), pool.dev_seq(0), out, 1, n - 1, Hq, 1 / 16, gate=dev(gate))
-    check(out.cpu().numpy(), ref, "config 2")
+    check(out.cpu().numpy(), ref, "config 2", flat=True)
     # device-resident position: same bits
     out2 = torch.empty_like(out)
     p1a.attn_decode_dev(dev(q), pool.dev_seq(0), out2, 1, dev(np.array([n - 1], np.int32)), n, Hq, 1 / 16, gate=dev(gate))
@@ -52,7 +52,7 @@ def test_config3_batched_8_slots(p1a):
     ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, 1 / 16, gate=gate)
     out = torch.empty((8, Hq, D), device="cuda")
     p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, 8, dev(pos), Hq, 1 / 16, gate=dev(gate))
-    check(out.cpu().numpy(), ref, "config 3")
+    check(out.cpu().numpy(), ref, "config 3", flat=True)
     for t in range(8):
         one = torch.empty((1, Hq, D), device="cuda")
         p1a.attn_decode(dev(q[t:t + 1]), pool.dev_seq(t), one, 1, int(pos[t]), Hq, 1 / 16, gate=dev(gate[t:t + 1]))
@@ -68,7 +68,7 @@ def test_config4_verify_4x4_q4_0_64k(p1a):
     ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, 1 / 16)
     out = torch.empty((4 * R, Hq, D), device="cuda")
     p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, 4 * R, dev(pos), Hq, 1 / 16, rows_per_seq=R)
-    check(out.cpu().numpy(), ref, "config 4")
+    check(out.cpu().numpy(), ref, "config 4", flat=True)
     for t in (0, 3, 6, 9, 15):                                  # verify rows == single-row calls
         one = torch.empty((1, Hq, D), device="cuda")
         p1a.attn_decode(dev(q[t:t + 1]), pool.dev_seq(t // R), one, 1, int(pos[t]), Hq, 1 / 16)
@@ -102,7 +102,7 @@ def test_config5_append_4096_then_prefill_over_32768(p1a):
     for a in range(0, T, 512):
         rows = np.arange(a, a + 512)
         ref = O.attn_rows(pool.host_seq(0), q[rows], (p0 + rows).astype(np.int32), Hq, 1 / 16, gate=gate[rows])
-        ma, rl = check(got[rows], ref, f"config 5 rows {a}..{a + 511}")
+        ma, rl = check(got[rows], ref, f"config 5 rows {a}..{a + 511}", flat=True)
         worst = (max(worst[0], ma), max(worst[1], rl))
         print(f"config 5: rows {a}..{a + 511} checked", flush=True)
     print(f"[parity] config 5, all {T} rows: worst block max_abs={worst[0]:.3e} rel_l2={worst[1]:.3e}")

@@ -267,3 +267,27 @@ def test_batched_rows_in_a_graph(p1a):
                 p1a.attn_decode_rows(q[t:t + 1], pool.devkv.with_rows(rt[t:t + 1]), one, 1, pos[t:t + 1], Hq, 1 / 16, gate=gate[t:t + 1])
                 s.synchronize()
                 assert torch.equal(one[0], out_g[t]), (back, t)
+
+
+def test_demoted_cache_on_a_fresh_stream_gets_the_scratch_it_needs(p1a):
+    """a cache the MFMA kernel cannot take (pages of 4 positions) goes to the generic kernel, which leaves four times the
+    partials per split stream; on a stream the library has not seen, after a release, the buffers it allocates must hold
+    them (they are sized from the call's own need as well as from the head shape's footprint), and a negative row
+    position reads no stream at all"""
+    Hq, Hkv, D, psh, T = 4, 4, 256, 2, 9
+    n = 300
+    p1a.lib().p1a_release()
+    pool = Pool(p1a, O.KV_Q4_0, Hq, Hkv, D, psh, [n], seed=131)
+    c = pool.dev_seq(0)
+    need = p1a.decode_scratch_bytes(c.struct(), Hq, T, 1)
+    assert need <= p1a.decode_footprint_bytes(Hq, Hkv, D)
+    q, _, _, gate = I.qkv(132, 1, T, Hq, Hkv, D)
+    ref = O.attn_rows(pool.host_seq(0), q, (n - T + np.arange(T)).astype(np.int32), Hq, 1 / 16, gate=gate)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        out = torch.zeros((T, Hq, D), device="cuda")
+        guard = torch.full((1 << 22,), 7.0, device="cuda")          # allocated right behind: must stay as it is
+        p1a.attn_decode(dev(q), c, out, T, n - T, Hq, 1 / 16, gate=dev(gate))
+        s.synchronize()
+    check(out.cpu().numpy(), ref, "generic kernel on a fresh stream")
+    assert bool((guard == 7.0).all())
