@@ -14,10 +14,13 @@
 namespace p1a {
 namespace {
 
+// the maximum over the 8 lanes of a block, in every one of them: lane ^ 1, lane ^ 2 within the quad, then the mirrored
+// half row (quad 0 <-> quad 1 of the 8) - on the data-parallel-primitive path, no LDS round trip; a maximum does not
+// care about the order it is taken in
 __device__ __forceinline__ float xor8_max(float a) {
-    a = fmaxf(a, __shfl_xor(a, 1));
-    a = fmaxf(a, __shfl_xor(a, 2));
-    a = fmaxf(a, __shfl_xor(a, 4));
+    a = max_dpp<0xB1>(a);     // quad_perm [1, 0, 3, 2]
+    a = max_dpp<0x4E>(a);     // quad_perm [2, 3, 0, 1]
+    a = max_dpp<0x141>(a);    // row_half_mirror
     return a;
 }
 
