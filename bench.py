@@ -147,7 +147,8 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
     # the caller-scratch variant (what attn_fold callers get): the cache is converted to f16 once per call
     scr = torch.empty(p1a.prefill_scratch_bytes(T, p0, Hq, Hkv, D), dtype=torch.uint8, device="cuda")
     # (eight untimed calls first: the first few calls after the pool has been built run 3 - 5 % slow, whichever variant they are)
-    sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate, scratch=scr), reps=5, warmup=8)
+    # (the part's clock settles over the first ten or so calls of a burst - every variant runs up to 10 % slow until then)
+    sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate, scratch=scr), reps=9, warmup=12)
     flop = 4.0 * D * Hq * (p0 * T + T * (T + 1) / 2)
     ex["prefill_T4096_p28672_q8_0_ms"] = round(sec * 1e3, 4)
     ex["prefill_TFLOPs"] = round(flop / sec / 1e12, 1)
@@ -155,10 +156,21 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
     ex["prefill_scratch_MB"] = round(scr.numel() / 1e6, 1)
     top["roofline_prefill"] = {
         "bound": "mfma", "achieved": round(flop / sec / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-        "frac": round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None, "kernel": "prefill_k<f16, 256, grouped, lds-direct>",
+        "frac": round(flop / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "traffic": prefill_traffic(), "kernel": "prefill_k<f16, 256, grouped, lds-direct>",
         "call_ms": round(sec * 1e3, 4),
         "note": "configs[4]: T = 4096 after 28672 tokens, q8_0, fused gate; flops = 4 D Hq (p0 T + T (T + 1) / 2); time = the "
-                "whole p1a_attn_prefill call with caller scratch (the convert-once pass of about 40 us included), median of 5"}
+                "whole p1a_attn_prefill call with caller scratch (the convert-once pass of about 40 us included), median of 9 "
+                "after 12 untimed calls; traffic = HBM-side bytes per call read from the committed rocprofv3 counter summary "
+                "(profiles/prefill_f16_staged_cfg5_traffic.json), not measured in this run"}
+    # a reference point for the bound: what a plain dense f16 GEMM of the vendor library (8192^3, fp32 accumulate) reaches
+    # on this part in the same run - the matrix pipe's practical ceiling under this part's power limit
+    ga = torch.randn((8192, 8192), device="cuda", dtype=torch.float16)
+    gb_ = torch.randn((8192, 8192), device="cuda", dtype=torch.float16)
+    gsec = time_eager(torch, lambda: torch.matmul(ga, gb_), reps=9, warmup=12)
+    ex["vendor_gemm_f16_8192_TFLOPs"] = round(2.0 * 8192 ** 3 / gsec / 1e12, 1)
+    ex["vendor_gemm_f16_frac_of_mfma_peak"] = round(2.0 * 8192 ** 3 / gsec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)
+    top["roofline_prefill"]["vendor_gemm_f16_frac"] = ex["vendor_gemm_f16_frac_of_mfma_peak"]
+    del ga, gb_
     out_scr = out.clone()
     sec = time_eager(torch, lambda: p1a.attn_prefill(q, c, out, T, p0, Hq, scale, gate=gate), reps=5)
     ex["prefill_no_scratch_ms"] = round(sec * 1e3, 4)                      # (the library's own staging copy: the reference's attn_prefill call site)
@@ -230,6 +242,14 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
     return ex
 
 
+def prefill_traffic():
+    tpath = os.path.join(ROOT, "profiles", "prefill_f16_staged_cfg5_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            return json.load(f).get("hbm_bytes_per_call")
+    return None
+
+
 def verify_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
     """configs[3]: MTP verify, 4 sequences x 4 rows (causal inside the block), q4_0, ctx 65536, each sequence's KV read once"""
     n4 = 65536
@@ -249,7 +269,12 @@ def verify_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
         sec_k = time_graph(torch, stream, [lambda: p1a.bench_decode_split_only(q, cr, out, 16, 0, Hq, scale, pos=pos, rows_per_seq=4)] * reps, 2)
     vb = 4 * n4 * 2 * p1a.kv_row_bytes(p1a.KV_Q4_0, Hkv, D)
     return {"verify_4x4_q4_0_64K_us": round(sec * 1e6, 2), "verify_GBs": round(vb / sec / 1e9, 1),
-            "verify_kernel_us": round(sec_k * 1e6, 2), "verify_kernel_frac_of_hbm_peak": round(vb / sec_k / 1e9 / HBM_PEAK_GBS, 4)}
+            "verify_kernel_us": round(sec_k * 1e6, 2), "verify_kernel_frac_of_hbm_peak": round(vb / sec_k / 1e9 / HBM_PEAK_GBS, 4),
+            "roofline_verify": {"bound": "hbm", "workload": "configs[3]: 4 sequences x 4 rows, q4_0, ctx 65536", "bytes": vb,
+                                "kernel": "dec_mfma_k<q4_0, 256, 2, 8>", "kernel_us": round(sec_k * 1e6, 2),
+                                "achieved": round(vb / sec_k / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                "frac": round(vb / sec_k / 1e9 / HBM_PEAK_GBS, 4), "call_us": round(sec * 1e6, 2),
+                                "call_frac": round(vb / sec / 1e9 / HBM_PEAK_GBS, 4)}}
 
 
 def batched_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
@@ -269,8 +294,14 @@ def batched_config(p1a, torch, stream, Hq, Hkv, D, psh, scale, reps=20):
     with torch.cuda.stream(stream):
         p1a.warmup(32, Hq, Hkv, D)
         sec = time_graph(torch, stream, [lambda: p1a.attn_decode_rows(q, cr, out, 8, pos, Hq, scale, gate=gate)] * reps, 2)
+        sec_k = time_graph(torch, stream, [lambda: p1a.bench_decode_split_only(q, cr, out, 8, 0, Hq, scale, pos=pos)] * reps, 2)
     bb = sum(lens) * 2 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, D)
-    res = {"batched_8slots_q8_0_us": round(sec * 1e6, 2), "batched_GBs": round(bb / sec / 1e9, 1), "batched_ctx": lens}
+    res = {"batched_8slots_q8_0_us": round(sec * 1e6, 2), "batched_GBs": round(bb / sec / 1e9, 1), "batched_ctx": lens,
+           "roofline_batched": {"bound": "hbm", "workload": "configs[2]: 8 slots, 1 row each, q8_0, ctx log-uniform in [1024, 32768]",
+                                "bytes": bb, "kernel": "dec_mfma_k<q8_0, 256, 1, 8, two workgroups per CU>",
+                                "kernel_us": round(sec_k * 1e6, 2), "achieved": round(bb / sec_k / 1e9, 1), "peak": HBM_PEAK_GBS,
+                                "unit": "GB/s", "frac": round(bb / sec_k / 1e9 / HBM_PEAK_GBS, 4), "call_us": round(sec * 1e6, 2),
+                                "call_frac": round(bb / sec / 1e9 / HBM_PEAK_GBS, 4)}}
     del kv, cr
     # the widest call the library takes: 32 slots, short contexts (2 K ... 5 K) - per-workgroup set-up is most of it
     lens32 = [2048 + 100 * i for i in range(32)]
@@ -554,6 +585,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(kgbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(kgbs / HBM_PEAK_GBS, 4), "traffic": traffic, "kernel": "dec_mfma_k<q8_0, 256, 1, 8>",
                      "kernel_us": round(sec_kernel * 1e6, 2),
+                     "call_us": round(sec * 1e6, 2), "call_frac": round(gbs / HBM_PEAK_GBS, 4),
                      "note": "achieved = algorithmic KV bytes of one launch (2 * ctx * 1088 B) / average duration of the "
                              "split-K kernel, event-timed on its stream over a graph of K launches walking the 8 layers (median of "
                              f"{REPLAYS} replays); traffic = HBM bytes per launch read from the committed rocprofv3 counter summary "
@@ -585,6 +617,9 @@ def main():
         res["extra"].update(extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, not args.no_cpu))
         if "roofline_prefill" in top:
             res["roofline_prefill"] = top["roofline_prefill"]
+        for key in ("roofline_verify", "roofline_batched"):
+            if key in res["extra"]:
+                res[key] = res["extra"].pop(key)
         if "cpu_prefill" in top:
             res["cpu_baseline"]["prefill"] = top["cpu_prefill"]
     print(json.dumps(res))

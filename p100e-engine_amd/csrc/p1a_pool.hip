@@ -16,15 +16,17 @@ namespace {
 
 using p1a::set_error;
 
+// One sequence of the pool. While it is resident it owns a row of the page table (its slot) and the pages listed here,
+// in position order; once offloaded it owns neither, only the host image of its pages and state.
 struct seq_t {
-    bool used = false;
-    int slot = -1;                    // page-table row / state slot (-1: offloaded)
-    int n_past = 0;
-    std::vector<int32_t> toks;        // processed tokens (size n_past)
-    std::vector<int32_t> pages;       // pool pages, position p in pages[p >> psh]
-    char * host = nullptr;            // offloaded: [pages][page_bytes] | state
-    int host_pages = 0;
-    size_t host_bytes = 0;
+    bool used = false;                // this entry of the sequence table is taken
+    int slot = -1;                    // resident: which page-table row and state block are its own; -1 while offloaded
+    int n_past = 0;                   // positions that hold KV (the next token goes to position n_past)
+    std::vector<int32_t> toks;        // the token ids behind those positions, one per position
+    std::vector<int32_t> pages;       // resident: pool page of every 2^psh positions, ascending by position
+    char * host = nullptr;            // offloaded: the image - page after page, each page_bytes, then the state block
+    int host_pages = 0;               // pages in that image
+    size_t host_bytes = 0;            // bytes of that image (counted against the pool's host budget)
 };
 
 }   // namespace
