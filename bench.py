@@ -208,19 +208,21 @@ def extras(p1a, torch, stream, Hq, Hkv, D, psh, scale, top, cpu):
         sec = time_graph(torch, stream, [lambda: p1a.attn_prep(qg4, kc, vc, w_q, w_k, pos4, q4, g4, c, p0, 4, Hq, 64, 1e7, 1e-6)] * 20, 2)
     ex["prep_4rows_q8_0_us"] = round(sec * 1e6, 2)
     del kv, c, q, gate, out
-    # a shape outside the MFMA kernels (q8_0 at head_dim 128: head rows are not whole 16-byte chunks): the generic
-    # one-wave-per-(stream, head, row) kernel, so that "correct, slow" has a number
-    kvg, ppg = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, 128, psh, 32768, 1, seed=25)
-    qg_ = normed((1, Hq, 128))
-    og_ = torch.empty((1, Hq, 128), device="cuda")
-    cg_ = kvg.slot(0, ppg)
-    with torch.cuda.stream(stream):
-        p1a.warmup(8, Hq, Hkv, 128)
-        sec = time_graph(torch, stream, [lambda: p1a.attn_decode(qg_, cg_, og_, 1, 32767, Hq, 1.0 / 128 ** 0.5)] * 20, 2)
-    gbytes = 2 * 32768 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, 128)
-    ex["generic_q8_0_D128_32K_us"] = round(sec * 1e6, 2)
-    ex["generic_q8_0_D128_32K_GBs"] = round(gbytes / sec / 1e9, 1)
-    del kvg, cg_
+    # q8_0 at head_dim 128 (head rows that are not whole 16-byte chunks): raw tiles fetched 4 bytes per lane and converted
+    # to f16 tiles by their wave, then the f16 MFMA kernel; and head_dim 96, which only the generic
+    # one-wave-per-(stream, head, row) kernel takes, so that "correct, slow" has a number
+    for Dx, tag in ((128, "staged_q8_0_D128_32K"), (96, "generic_q8_0_D96_32K")):
+        kvg, ppg = build_pool(p1a, torch, p1a.KV_Q8_0, Hq, Hkv, Dx, psh, 32768, 1, seed=25)
+        qg_ = normed((1, Hq, Dx))
+        og_ = torch.empty((1, Hq, Dx), device="cuda")
+        cg_ = kvg.slot(0, ppg)
+        with torch.cuda.stream(stream):
+            p1a.warmup(8, Hq, Hkv, Dx)
+            sec = time_graph(torch, stream, [lambda: p1a.attn_decode(qg_, cg_, og_, 1, 32767, Hq, 1.0 / Dx ** 0.5)] * 20, 2)
+        gbytes = 2 * 32768 * p1a.kv_row_bytes(p1a.KV_Q8_0, Hkv, Dx)
+        ex[tag + "_us"] = round(sec * 1e6, 2)
+        ex[tag + "_GBs"] = round(gbytes / sec / 1e9, 1)
+        del kvg, cg_
     ex.update(verify_config(p1a, torch, stream, Hq, Hkv, D, psh, scale))
     ex.update(mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale))
     ex.update(mtp_verify_loop(p1a, torch, Hq, Hkv, D, psh, scale, graphed=True))

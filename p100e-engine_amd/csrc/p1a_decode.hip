@@ -55,6 +55,16 @@ template <uint32_t KT, int D> struct tile_cfg {
 };
 
 
+// Staged source (q8_0 / q4_0 head rows that are not whole 16-byte chunks, i.e. D = 64 or 128): the raw image of 16 head
+// rows is fetched 4 bytes per lane, converted by its wave into the f16 tile the f16 kernel reads, and computed on as f16.
+template <uint32_t KS, int D> struct raw_cfg {
+    static constexpr int HB = (int) head_bytes(KS, D);
+    static constexpr int RAW_B = 16 * HB;                      // the linear image of 16 raw head rows
+    static constexpr int NDW = RAW_B / 4;
+    static constexpr int NRND = (NDW + 63) / 64;               // load rounds per tile (4 bytes per lane)
+    static_assert(HB % 4 == 0, "raw head rows are whole dwords");
+};
+
 struct dec_params {
     const float * q;
     const char * kc;
@@ -126,6 +136,10 @@ __device__ __forceinline__ void dma16(const char * sbase, uint32_t voff, uint32_
 __device__ __forceinline__ void dma16v(const char * vaddr, uint32_t lds) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" :: "v"(vaddr), "s"(lds) : "memory", "m0");
 }
+// 4 bytes per lane: lane i lands at M0 + 4 i
+__device__ __forceinline__ void dma4(const char * sbase, uint32_t voff, uint32_t lds) {
+    asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dword %0, %1" :: "v"(voff), "s"(sbase), "s"(__builtin_amdgcn_readfirstlane((int) lds)) : "memory", "m0");
+}
 template <int N> __device__ __forceinline__ void wait_vm_imm() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 // wait until at most `newer` tile fetches (NR loads each) issued after the wanted one are still in flight
 template <int NR> __device__ __forceinline__ void wait_tiles(int newer) {
@@ -147,23 +161,31 @@ __device__ __forceinline__ int sload_i32(const int32_t * p) {
 // the fold and the memory round trips of the first. Tile t + 1 of K is then requested once the products with tile t of K
 // are done, V likewise; everything a lane computes, and the order it computes it in, is the same as in the double-buffered
 // kernel, so the partials are the same bits. One column tile only (NT == 1, at most 16 live columns).
-template <uint32_t KT, int D, int NT, int NWV, bool SB>
+// KS (when it differs from KT = f16): the type the cache holds - its raw tiles are staged (raw_cfg) and converted to f16
+template <uint32_t KT, int D, int NT, int NWV, bool SB, uint32_t KS = KT>
 __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const dec_params P) {
     using C = tile_cfg<KT, D>;
+    using RW = raw_cfg<KS, D>;
+    constexpr bool STG = KS != KT;
     static_assert(!SB || NT == 1, "the single-buffered variant has one column tile");
+    static_assert(!STG || (KT == P1A_KV_F16 && !SB && D <= 128), "staged tiles are converted to f16 and take the double-buffered build");
+    constexpr int NLD = STG ? RW::NRND : C::NRND;             // vector-memory operations per tile fetch
+    // STG: slot array 0 = the f16 K tile of every wave, 1 = the f16 V tile, 2 = two raw K tiles, 3 = two raw V tiles
+    constexpr int SLOTX = STG ? (C::SLOT_B > 2 * RW::RAW_B ? C::SLOT_B : 2 * RW::RAW_B) : C::SLOT_B;
     // four tile slots per wave (K and V, two each), plus a small per-wave table. SB: one pool that holds one K slot, one
     // V slot (and the q4_0 copy) per wave at the size of a tile, and is handed over to the fold as a whole afterwards:
     // wave w parks 8 columns at a time, dim quarter k at PARK_B (4 w + k)
-    constexpr int SLB = SB ? C::TILE_B : C::SLOT_B;            // bytes per slot
+    constexpr int SLB = SB ? C::TILE_B : SLOTX;                // bytes per slot
     constexpr int PARK_B = 8 * C::QDP * 4;                     // SB: one dim quarter of 8 parked columns
     constexpr int POOL_T = NWV * (2 * C::TILE_B + C::VA_B), POOL_P = NWV * 4 * PARK_B;
     __shared__ __attribute__((aligned(16))) char pool[SB ? (POOL_T > POOL_P ? POOL_T : POOL_P) : 16];
     // (one array, slot array k at k NWV SLOT_B: K slot 0, K slot 1, V slot 0, V slot 1 - the fold addresses them by number)
-    __shared__ __attribute__((aligned(16))) char slots[SB ? 16 : 4 * NWV * C::SLOT_B];
+    __shared__ __attribute__((aligned(16))) char slots[SB ? 16 : 4 * NWV * SLOTX];
     __shared__ __attribute__((aligned(16))) char qown[SB ? 16 * C::QRS : 16];          // SB: the f16 Q table (first the fp32 copy of up to 8 rows)
-    char * const kb0 = SB ? pool : slots, * const vb0 = SB ? pool + NWV * C::TILE_B : slots + 2 * NWV * C::SLOT_B;
-    char * const kb1 = SB ? kb0 : slots + NWV * C::SLOT_B, * const vb1 = SB ? vb0 : slots + 3 * NWV * C::SLOT_B;
-    static_assert(SB || (32 * D * 4 <= NWV * C::SLOT_B && 32 * C::QRS <= NWV * C::SLOT_B), "the Q copies (at most 32 columns) fit over the second K and V slots");
+    // (STG: "K slot 1" / "V slot 1" - where the Q copies go before any tile is converted - are the f16 tile arrays themselves)
+    char * const kb0 = SB ? pool : slots, * const vb0 = SB ? pool + NWV * C::TILE_B : STG ? slots + NWV * SLOTX : slots + 2 * NWV * SLOTX;
+    char * const kb1 = SB || STG ? kb0 : slots + NWV * SLOTX, * const vb1 = SB || STG ? vb0 : slots + 3 * NWV * SLOTX;
+    static_assert(SB || (32 * D * 4 <= NWV * SLOTX && 32 * C::QRS <= NWV * SLOTX), "the Q copies (at most 32 columns) fit over the second K and V slots");
     static_assert(!SB || 8 * D * 4 <= 16 * C::QRS, "SB: the fp32 copy of 8 rows fits where the f16 table of 16 goes");
     // q8_0 with two column tiles has no registers left for 64 dwords of Q operands (spills there cost more than their
     // traffic: the compiler can only wait for a reload with "no vector memory operation outstanding", tiles included):
@@ -213,6 +235,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     char * const vs0 = vb0 + wave * SLB, * const vs1 = vb1 + wave * SLB;
     char * const tab = tabs + wave * C::TAB_B;
     char * const va = (SB ? pool + 2 * NWV * C::TILE_B : vab) + wave * C::VA_B;
+    char * const rawk = slots + (2 * NWV + wave) * SLOTX, * const rawv = slots + (3 * NWV + wave) * SLOTX;   // STG: two raw tiles each
 
     // column -> row of the group (at most 4 rows: three comparisons instead of a division)
     auto row_of = [&](int col) { return (col >= P.GQA) + (col >= 2 * P.GQA) + (col >= 3 * P.GQA); };
@@ -255,16 +278,18 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     // "nothing outstanding", and placed after the requests such a wait would also wait for the tiles.
 #pragma unroll
     for (int r = 0; r < NT; ++r) asm volatile("" : "+v"(plim[r]));
-    const size_t head_off = (size_t) hk * C::HB;
+    const size_t head_off = (size_t) hk * (STG ? RW::HB : C::HB);
     const int rowb = (int) P.pg.rowb;
 
     // chunk i = 64 * round + lane of a tile is bytes [16 cir, +16) of key i / CPK; static per-lane source offsets
-    unsigned soff[C::NRND];
+    // (STG: dword i of the raw image is dword i % (HB / 4) of key i / (HB / 4))
+    constexpr int IPK = STG ? RW::HB / 4 : C::CPK, ISZ = STG ? 4 : 16;     // items per key, bytes per item
+    unsigned soff[NLD];
 #pragma unroll
-    for (int rd = 0; rd < C::NRND; ++rd) {
+    for (int rd = 0; rd < NLD; ++rd) {
         const int i = rd * 64 + lane;
-        const int key = i / C::CPK, cir = i - key * C::CPK;
-        soff[rd] = (unsigned) (key * rowb + (int) head_off + cir * 16);
+        const int key = i / IPK, cir = i - key * IPK;
+        soff[rd] = (unsigned) (key * rowb + (int) head_off + cir * ISZ);
     }
 
     // Tile t of this wave (t = 0, 1, ...): unit split + (t >> 1) * nsplit, keys [ts, ts + 16) with
@@ -286,11 +311,53 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                 asm volatile("" : "+v"(ii));
                 off -= (uint32_t) (max(ii / C::CPK - last, 0) * rowb);
             } else {
-                const int key = i / C::CPK, cir = i - key * C::CPK;
-                off = (uint32_t) (min(key, last) * rowb + (int) head_off + cir * 16);
+                const int key = i / IPK, cir = i - key * IPK;
+                off = (uint32_t) (min(key, last) * rowb + (int) head_off + cir * ISZ);
             }
         }
-        if (C::NCH % 64 == 0 || i < C::NCH) dma16(b0, off, lds_addr(slot) + rd * 1024);
+        if constexpr (STG) { if (RW::NDW % 64 == 0 || i < RW::NDW) dma4(b0, off, lds_addr(slot) + rd * 256); }
+        else if (C::NCH % 64 == 0 || i < C::NCH) dma16(b0, off, lds_addr(slot) + rd * 1024);
+    };
+    // STG: the raw image of 16 head rows at `raw` -> the f16 tile at `dst` (row c at c * 2 D bytes), by this wave alone. The
+    // values are code * f16 scale rounded once to f16 - what the D = 256 kernels feed their products and the prefill stages.
+    auto convert = [&](const char * raw, char * dst) {
+        if constexpr (STG && KS == P1A_KV_Q8_0) {
+            // item = 8 codes of one key: D / 8 items per key; codes start behind the D / 32 scales
+            constexpr int IPR = D / 8, NIT = 16 * IPR / 64;
+#pragma unroll
+            for (int x = 0; x < NIT; ++x) {
+                const int it = x * 64 + lane, key = it / IPR, p8 = it - key * IPR;
+                const char * row = raw + key * RW::HB;
+                const uint32_t * cw = reinterpret_cast<const uint32_t *>(row + (D / 32) * 2 + 8 * p8);   // (4-byte aligned)
+                const uint32_t w0 = cw[0], w1 = cw[1];
+                const uint32_t d16 = *reinterpret_cast<const uint16_t *>(row + 2 * (p8 >> 2));
+                const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
+                const u2 a = deq4(w0, dd, dd), b = deq4(w1, dd, dd);
+                *reinterpret_cast<u4 *>(dst + key * (2 * D) + 16 * p8) = u4{a.lo, a.hi, b.lo, b.hi};
+            }
+        } else if constexpr (STG) {
+            // item = one 18-byte block of one key (2-byte aligned): values 0 .. 15 are its low nibbles, 16 .. 31 the high ones
+            constexpr int BPR = D / 32, NIT = (16 * BPR + 63) / 64;
+#pragma unroll
+            for (int x = 0; x < NIT; ++x) {
+                const int it = x * 64 + lane, key = it / BPR, b = it - key * BPR;
+                if (16 * BPR % 64 == 0 || it < 16 * BPR) {
+                    const uint16_t * blk = reinterpret_cast<const uint16_t *>(raw + key * RW::HB + 18 * b);
+                    const uint32_t d16 = blk[0];
+                    const h2 dd = __builtin_bit_cast(h2, d16 | (d16 << 16));
+                    u4 lo[2], hi[2];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t w = (uint32_t) blk[1 + 2 * q] | ((uint32_t) blk[2 + 2 * q] << 16);
+                        const u2 l = deq4n(w & 0x0f0f0f0fu, dd), h = deq4n((w >> 4) & 0x0f0f0f0fu, dd);
+                        lo[q >> 1][2 * (q & 1)] = l.lo; lo[q >> 1][2 * (q & 1) + 1] = l.hi;
+                        hi[q >> 1][2 * (q & 1)] = h.lo; hi[q >> 1][2 * (q & 1) + 1] = h.hi;
+                    }
+                    u4 * o = reinterpret_cast<u4 *>(dst + key * (2 * D) + 64 * b);
+                    o[0] = lo[0]; o[1] = lo[1]; o[2] = hi[0]; o[3] = hi[1];
+                }
+            }
+        }
     };
     auto page_of = [&](int ts) -> const int32_t * { return ptab + (ts >> P.pg.psh); };
 
@@ -303,12 +370,12 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
         if (ptab && (!first || (tile_start(0) >> P.pg.psh) != idx_early)) pg0 = sload_i32(page_of(tile_start(0)));
         off0 = tile_off(tile_start(0), pg0);
 #pragma unroll
-        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ks0, P.kc + off0, tile_start(0), rd);
+        for (int rd = 0; rd < NLD; ++rd) fetch_round(STG ? rawk : ks0, P.kc + off0, tile_start(0), rd);
     };
     auto request_v0 = [&]() {
         if (tile_start(0) >= n_max) return;
 #pragma unroll
-        for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vs0, P.vc + off0, tile_start(0), rd);
+        for (int rd = 0; rd < NLD; ++rd) fetch_round(STG ? rawv : vs0, P.vc + off0, tile_start(0), rd);
     };
     // This wave's share of the Q rows -> LDS (fp32, column col at col * 4 D bytes of K slot 1; lane i brings floats
     // 4 i .. 4 i + 3). These requests are OLDER than the tile requests that follow, so waiting for them below does not
@@ -349,7 +416,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     // piece - into an f16 table over V slot 1 (rows padded: conflict-free reads), and every lane picks its operands
     // out of that. (While a workgroup's requests queue up at the memory pipeline a wave cannot issue anything else:
     // what little work there is before the first tile is best kept short.)
-    if (!q_direct) { if (tile_start(0) < n_max) wait_vm_imm<2 * C::NRND>(); else wait_vm_imm<0>(); }
+    if (!q_direct) { if (tile_start(0) < n_max) wait_vm_imm<2 * NLD>(); else wait_vm_imm<0>(); }
     __syncthreads();
     char * const qt = SB ? qown : QLDS ? qtab : vb1;
     if constexpr (SB) {   // in place (8 columns): every piece is read, by the thread that will write it, before any is written
@@ -414,7 +481,9 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     }
 
     // one 16-key tile from slots (ks, vs); the loads of tile t + 1 into (ksn, vsn) are issued between its products
-    auto step = [&](char * ks, char * vs, char * ksn, char * vsn, int t) {
+    auto step = [&](char * ks, char * vs, char * ksn_, char * vsn_, int t) {
+        // (STG: ks / vs are the wave's f16 tiles; the raw tiles alternate between the two halves of its raw areas)
+        char * const ksn = STG ? rawk + ((t + 1) & 1) * RW::RAW_B : ksn_, * const vsn = STG ? rawv + ((t + 1) & 1) * RW::RAW_B : vsn_;
         const int ts = tile_start(t);
         const int tn = tile_start(t + 1);
         const bool have_n = tn < n_max;
@@ -423,7 +492,8 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
         if ((t ^ (wave >> 2)) & 1) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0);
         int pgn = 0;
         if (ptab && have_n) pgn = sload_i32(page_of(tn));
-        wait_vm_imm<C::NRND>();                               // K of tile t has landed (only its V is younger)
+        wait_vm_imm<NLD>();                                   // K of tile t has landed (only its V is younger)
+        if constexpr (STG) convert(rawk + (t & 1) * RW::RAW_B, ks);
         const size_t on = have_n ? tile_off(tn, pgn) : 0;
         const char * const kn = P.kc + on, * const vn = P.vc + on;
         // ---- S^T = K Q^T ----
@@ -442,7 +512,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                     else qo = qf[r][m];
                     s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, qo, s[r], 0, 0, 0);
                 }
-                if (!SB && have_n && m < C::NRND) fetch_round(ksn, kn, tn, m);
+                if (!SB && have_n && m < NLD) fetch_round(ksn, kn, tn, m);
             }
         } else if constexpr (KT == P1A_KV_Q4_0) {   // 8 blocks of 18 B: f16 scale, then 16 nibble bytes (2-byte aligned)
             // nibble bytes 4 g .. 4 g + 3 of block b sit at 18 b + 2 + 4 g: a whole dword in odd blocks, the upper and
@@ -475,7 +545,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                     } else qo = qf[r][b];
                     s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a), qo, s[r], 0, 0, 0);
                 }
-                if (!SB && have_n && b < C::NRND) fetch_round(ksn, kn, tn, b);
+                if (!SB && have_n && b < NLD) fetch_round(ksn, kn, tn, b);
                 kcur = knxt;
             }
         } else {   // q8_0: 16 B of scales, then 16 chunks of 16 codes
@@ -502,17 +572,17 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                     s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a0), q0, s[r], 0, 0, 0);
                     s[r] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, a1), q1, s[r], 0, 0, 0);
                 }
-                if (!SB && have_n && jj < C::NRND) fetch_round(ksn, kn, tn, jj);
+                if (!SB && have_n && jj < NLD) fetch_round(ksn, kn, tn, jj);
             }
         }
         if (!SB && have_n) {   // the rounds the product loop had no place for
 #pragma unroll
-            for (int rd = (KT == P1A_KV_Q8_0 ? C::NMF / 2 : C::NMF); rd < C::NRND; ++rd) fetch_round(ksn, kn, tn, rd);
+            for (int rd = (KT == P1A_KV_Q8_0 ? C::NMF / 2 : C::NMF); rd < NLD; ++rd) fetch_round(ksn, kn, tn, rd);
         }
         if (SB && have_n) {    // the K slot is free once its last fragment has been read
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-            for (int rd = 0; rd < C::NRND; ++rd) fetch_round(ksn, kn, tn, rd);
+            for (int rd = 0; rd < NLD; ++rd) fetch_round(ksn, kn, tn, rd);
         }
 
         // ---- online softmax (log2 domain); column = query row, this lane holds keys ts + 4 g + i ----
@@ -552,7 +622,8 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
             }
         }
 
-        if (have_n) wait_vm_imm<C::NRND>(); else wait_vm_imm<0>();   // V of tile t has landed (only K of t + 1 is younger)
+        if (have_n) wait_vm_imm<NLD>(); else wait_vm_imm<0>();   // V of tile t has landed (only K of t + 1 is younger)
+        if constexpr (STG) convert(rawv + (t & 1) * RW::RAW_B, vs);
         // ---- O^T += V^T P^T: k-slot i of lane group g is key ts + 4 g + i, the key of this lane's P value i ----
         if constexpr (KT == P1A_KV_F16) {
             const int kk = c >> 2, jq = c & 3;
@@ -563,7 +634,11 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                 const h4 a = __builtin_bit_cast(h4, w);
 #pragma unroll
                 for (int r = 0; r < NT; ++r) o[r][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, pb[r], o[r][j], 0, 0, 0);
-                if (!SB && have_n && j < C::NRND) fetch_round(vsn, vn, tn, j);
+                if (!SB && have_n && j < NLD) fetch_round(vsn, vn, tn, j);
+            }
+            if (!SB && have_n) {   // (staged tiles can take more rounds than the loop has places)
+#pragma unroll
+                for (int rd = C::NDT; rd < NLD; ++rd) fetch_round(vsn, vn, tn, rd);
             }
         } else if constexpr (KT == P1A_KV_Q4_0) {
             {   // re-align: nibble bytes of block bb of a key -> va[key][bb][16] (8-byte aligned for the transposing read);
@@ -618,7 +693,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                         o[r][2 * b + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a1), pb[r], o[r][2 * b + 1], 0, 0, 0);
                     }
                 }
-                if (!SB && have_n && p < C::NRND) fetch_round(vsn, vn, tn, p);
+                if (!SB && have_n && p < NLD) fetch_round(vsn, vn, tn, p);
             }
         } else {
             {   // transposed scale table tab[block][key] (f16, 32 B per block)
@@ -649,14 +724,14 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
                     o[r][j] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a0), pb[r], o[r][j], 0, 0, 0);
                     o[r][j + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h4, a1), pb[r], o[r][j + 1], 0, 0, 0);
                 }
-                if (!SB && have_n && j / 2 < C::NRND) fetch_round(vsn, vn, tn, j / 2);
+                if (!SB && have_n && j / 2 < NLD) fetch_round(vsn, vn, tn, j / 2);
             }
         }
-        static_assert(C::NRND <= (KT == P1A_KV_F16 ? C::NDT : KT == P1A_KV_Q8_0 ? C::NDT / 2 : C::NMF / 2), "the PV loop must have room for every V load");
+        static_assert(KT == P1A_KV_F16 || NLD <= (KT == P1A_KV_Q8_0 ? C::NDT / 2 : C::NMF / 2), "the PV loop must have room for every V load");
         if (SB && have_n) {    // the V slot likewise
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-            for (int rd = 0; rd < C::NRND; ++rd) fetch_round(vsn, vn, tn, rd);
+            for (int rd = 0; rd < NLD; ++rd) fetch_round(vsn, vn, tn, rd);
         }
 #pragma unroll
         for (int r = 0; r < NT; ++r) ol[r] = __builtin_amdgcn_mfma_f32_16x16x16f16(ones, pb[r], ol[r], 0, 0, 0);
@@ -678,7 +753,7 @@ __global__ void __launch_bounds__(NWV * 64, SB ? NWV / 2 : 1) dec_mfma_k(const d
     const int c_f = tid_f & 15, g_f = (tid_f >> 4) & 3;
     auto park = [&](int w, int k) -> float * {                // dim quarter k of wave w
         if constexpr (SB) return reinterpret_cast<float *>(pool + (4 * w + k) * PARK_B);
-        else return reinterpret_cast<float *>(slots + (k * NWV + w) * C::SLOT_B);
+        else return reinterpret_cast<float *>(slots + (k * NWV + w) * SLOTX);
     };
 #pragma unroll
     for (int r = 0; r < NT; ++r) {
@@ -941,8 +1016,10 @@ __global__ void __launch_bounds__(256) sigmoid_mul_k(float * __restrict__ x, con
 }
 
 // ---- launch plan: which kernel a shape takes, and how the keys are split ----
-// The MFMA kernel needs 16-byte aligned head rows (f16: D in {64, 128, 256}; q8_0: D == 256), 16-byte aligned
-// bases and strides, pages of >= 16 positions and GQA <= 16. Everything else takes the generic kernel.
+// The MFMA kernel needs 16-byte aligned head rows (f16: D in {64, 128, 256}; q8_0 / q4_0: D == 256), 16-byte aligned
+// bases and strides, pages of >= 16 positions and GQA <= 16; q8_0 / q4_0 at D = 64 or 128 (head rows of whole dwords)
+// take its staged build, which fetches 4 bytes per lane and only needs 4-byte alignment. Everything else takes the
+// generic kernel.
 struct dec_plan {
     bool mfma;
     int GQA, NW, NT, RG;
@@ -952,10 +1029,11 @@ struct dec_plan {
 
 bool mfma_ok(const p1a_kv & c, int GQA) {
     if (GQA < 1 || GQA > 16) return false;
-    if (c.type == P1A_KV_F16) { if (c.D != 64 && c.D != 128 && c.D != 256) return false; }
-    else { if (c.D != 256) return false; }   // q8_0 / q4_0 head rows are whole 16-byte chunks only at D = 256
-    if (((uintptr_t) c.k | (uintptr_t) c.v) & 15) return false;
-    if (c.pt && ((c.pstride & 15) || c.psh < 4)) return false;
+    if (c.D != 64 && c.D != 128 && c.D != 256) return false;
+    const bool staged = c.type != P1A_KV_F16 && c.D != 256;   // q8_0 / q4_0 head rows are whole 16-byte chunks only at D = 256
+    const uintptr_t al = staged ? 3 : 15;
+    if (((uintptr_t) c.k | (uintptr_t) c.v) & al) return false;
+    if (c.pt && ((c.pstride & al) || c.psh < 4)) return false;
     return true;
 }
 
@@ -991,7 +1069,7 @@ void finish_plan(dec_plan & p) {
     if (p.mfma) p.NS = p.nsplit;
 }
 
-template <uint32_t KT, int D>
+template <uint32_t KT, int D, uint32_t KS = KT>
 int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hipStream_t s) {
     dec_params P;
     P.q = a.q; P.kc = (const char *) c.k; P.vc = (const char *) c.v;
@@ -1009,10 +1087,13 @@ int launch_mfma(const p1a_kv & c, const decode_args & a, const dec_plan & pl, hi
     // (A workgroup walks ONE split stream whatever the call: letting it walk several in turn - fewer, longer workgroups
     // for calls of many - measured slower on every shape tried, e.g. 8 x 4 rows q4_0 at 8 K 72 -> 60 us with one.)
     const long long wgs_all = (long long) pl.nsplit * c.Hkv * ((a.T + pl.RG - 1) / pl.RG);
-    const bool sb = pl.NT == 1 && wgs_all >= 2LL * (a.cus > 0 ? a.cus : 256);
+    const bool sb = KS == KT && pl.NT == 1 && wgs_all >= 2LL * (a.cus > 0 ? a.cus : 256);
     const dim3 grid(pl.nsplit * c.Hkv, (a.T + pl.RG - 1) / pl.RG);
-#define P1A_DEC(NT_, NW_) dec_mfma_k<KT, D, NT_, NW_, false><<<grid, NW_ * 64, 0, s>>>(P)
-    if constexpr (big_tiles) {
+#define P1A_DEC(NT_, NW_) dec_mfma_k<KT, D, NT_, NW_, false, KS><<<grid, NW_ * 64, 0, s>>>(P)
+    if constexpr (KS != KT) {
+        if (pl.NT == 1) P1A_DEC(1, 8);
+        else P1A_DEC(2, 8);
+    } else if constexpr (big_tiles) {
         if (sb) dec_mfma_k<KT, D, 1, 4, true><<<grid, 256, 0, s>>>(P);
         else if (pl.NT == 1) P1A_DEC(1, 4);
         else P1A_DEC(2, 4);
@@ -1054,8 +1135,12 @@ int launch_decode(const p1a_kv & c, const decode_args & a, hipStream_t s) {
     }
     int rc;
     if (pl.mfma) {
-        if (c.type == P1A_KV_Q8_0) rc = launch_mfma<P1A_KV_Q8_0, 256>(c, a, pl, s);
-        else if (c.type == P1A_KV_Q4_0) rc = launch_mfma<P1A_KV_Q4_0, 256>(c, a, pl, s);
+        if (c.type == P1A_KV_Q8_0 && c.D == 256) rc = launch_mfma<P1A_KV_Q8_0, 256>(c, a, pl, s);
+        else if (c.type == P1A_KV_Q4_0 && c.D == 256) rc = launch_mfma<P1A_KV_Q4_0, 256>(c, a, pl, s);
+        else if (c.type == P1A_KV_Q8_0 && c.D == 128) rc = launch_mfma<P1A_KV_F16, 128, P1A_KV_Q8_0>(c, a, pl, s);
+        else if (c.type == P1A_KV_Q8_0) rc = launch_mfma<P1A_KV_F16, 64, P1A_KV_Q8_0>(c, a, pl, s);
+        else if (c.type == P1A_KV_Q4_0 && c.D == 128) rc = launch_mfma<P1A_KV_F16, 128, P1A_KV_Q4_0>(c, a, pl, s);
+        else if (c.type == P1A_KV_Q4_0) rc = launch_mfma<P1A_KV_F16, 64, P1A_KV_Q4_0>(c, a, pl, s);
         else if (c.D == 256) rc = launch_mfma<P1A_KV_F16, 256>(c, a, pl, s);
         else if (c.D == 128) rc = launch_mfma<P1A_KV_F16, 128>(c, a, pl, s);
         else rc = launch_mfma<P1A_KV_F16, 64>(c, a, pl, s);

@@ -362,3 +362,37 @@ def test_standalone_gate_equals_the_fused_one(p1a):
     assert np.abs(got - want).max() <= 1e-6 * max(1.0, np.abs(want).max())
     assert np.array_equal(got[0, :64], 0.5 * ungated.reshape(3, -1)[0, :64])
     assert np.all(got[1, [0]] == 0.0 * ungated.reshape(3, -1)[1, [0]])       # sigmoid(-200) = 0: expf overflows to inf, 1 / inf = 0
+
+
+@pytest.mark.parametrize("kv_type,Hq,Hkv,D", [(O.KV_Q8_0, 24, 4, 128), (O.KV_Q4_0, 24, 4, 128), (O.KV_Q8_0, 16, 2, 64),
+                                              (O.KV_Q4_0, 8, 2, 64), (O.KV_Q8_0, 32, 2, 128)])
+def test_staged_tiles_for_small_heads(p1a, kv_type, Hq, Hkv, D):
+    """q8_0 / q4_0 head rows at D = 64 or 128 are not whole 16-byte chunks; their raw tiles are fetched 4 bytes per lane,
+    converted to f16 tiles by the wave that owns them and multiplied on the matrix pipe like an f16 cache (the reference
+    refuses these shapes, src/fast/attn_dec2.cu:493). Every depth class against the oracle - one key, a ragged last tile,
+    a tile boundary, several units - for 1 ... 4 rows (one and two column tiles); and the identities the D = 256 kernels keep:
+    paged == contiguous, row t of a T-row call == the T = 1 call, batched rows == single, all bit for bit."""
+    psh, n = 5, 2100
+    pool = Pool(p1a, kv_type, Hq, Hkv, D, psh, [n, 700], seed=300 + D)
+    cont = pool.dev_contiguous(0)
+    scale = 1.0 / np.sqrt(D)
+    for T, p0 in ((1, 0), (1, 14), (1, 15), (1, 16), (2, 255), (3, 511), (4, 1000), (1, n - 1), (4, n - 4)):
+        q, _, _, gate = I.qkv(400 + T + p0, 1, T, Hq, Hkv, D)
+        ref = O.attn_rows(pool.host_seq(0), q, (p0 + np.arange(T)).astype(np.int32), Hq, scale, gate=gate)
+        out = run_decode(p1a, pool.dev_seq(0), q, T, p0, Hq, scale, gate=gate)
+        check(out, ref, f"staged {kv_type} {Hq}/{Hkv}/{D} T {T} p0 {p0}")
+        assert np.array_equal(out, run_decode(p1a, cont, q, T, p0, Hq, scale, gate=gate)), (T, p0)      # paged == contiguous
+        for t in range(T):                                                                               # row t == the T = 1 call
+            one = run_decode(p1a, pool.dev_seq(0), q[t:t + 1], 1, p0 + t, Hq, scale, gate=gate[t:t + 1])
+            assert np.array_equal(one[0], out[t]), (T, p0, t)
+    # rows of two sequences in one call == each on its own
+    pos = np.array([n - 1, 699, 1234, 5], np.int32)
+    rtab = np.array([0, pool.maxp, 0, pool.maxp], np.int32)
+    q, _, _, gate = I.qkv(499, 1, 4, Hq, Hkv, D)
+    ref = O.attn_rows(pool.host.view(rtab=rtab), q, pos, Hq, scale, gate=gate)
+    out = torch.empty((4, Hq, D), device="cuda")
+    p1a.attn_decode_rows(dev(q), pool.devkv.with_rows(dev(rtab)), out, 4, dev(pos), Hq, scale, gate=dev(gate))
+    check(out.cpu().numpy(), ref, f"staged {kv_type} batched rows")
+    for t in range(4):
+        one = run_decode(p1a, pool.dev_seq(int(rtab[t] // pool.maxp)), q[t:t + 1], 1, int(pos[t]), Hq, scale, gate=gate[t:t + 1])
+        assert np.array_equal(one[0], out[t].cpu().numpy()), t

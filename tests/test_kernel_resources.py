@@ -41,10 +41,15 @@ def test_decode_kernels_fit_their_budget(tmp_path):
     for name, r in ks.items():
         assert r.get("VGPRs Spill", 0) == 0 and r.get("SGPRs Spill", 0) == 0, (name, r)
         assert r.get("ScratchSize", 0) == 0, (name, r)
-    # dec_mfma_k<KT, D, NT, NW, SB>: the mangled name ends ...ELi<NW>ELb<SB>EEEv...
-    sb = {k: v for k, v in ks.items() if re.search(r"ELb1EEEv", k)}
+    # dec_mfma_k<KT, D, NT, NW, SB, KS>: the mangled name ends ...ELi<NW>ELb<SB>ELj<KS>EEEv...
+    sb = {k: v for k, v in ks.items() if re.search(r"ELb1ELj\d+EEEv", k)}
     assert len(sb) >= 5, sorted(ks)
+    # the staged builds (KS != KT: q8_0 / q4_0 at D = 64, 128 converted to f16 tiles) are there, one workgroup per CU
+    staged = {k: v for k, v in ks.items() if re.search(r"ILj1ELi(64|128)ELi[12]ELi8ELb0ELj[28]EEEv", k)}
+    assert len(staged) == 8, sorted(ks)
+    for name, r in staged.items():
+        assert r["LDS Size"] <= 160 * 1024, (name, r)
     for name, r in sb.items():
-        waves = int(re.search(r"ELi(\d+)ELb1EEEv", name).group(1))
+        waves = int(re.search(r"ELi(\d+)ELb1ELj\d+EEEv", name).group(1))
         assert r["LDS Size"] <= 80 * 1024, (name, r)                       # two workgroups in 160 KB
         assert r["Occupancy"] * 4 >= 2 * waves, (name, r)                   # two workgroups' waves on the 4 SIMDs
