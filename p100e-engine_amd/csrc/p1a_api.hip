@@ -34,7 +34,7 @@ namespace {
 // old one only for later calls - the old one stays allocated (g_retired) until p1a_release(). Nothing is allocated
 // while the stream is being captured. The partials of a key-split prefill have a pair of their own.
 struct bufpair { float * o = nullptr; float * ml = nullptr; size_t cap_o = 0, cap_ml = 0; };
-struct stream_bufs { int dev = -1; hipStream_t s = nullptr; bufpair dec, pf; void * stage = nullptr; size_t cap_stage = 0; };
+struct stream_bufs { int dev = -1; hipStream_t s = nullptr; bufpair dec, pf; void * stage = nullptr; size_t cap_stage = 0; bool stage_captured = false; };
 constexpr int MAX_SCR = 64;
 constexpr int MAX_RETIRED = 1024;
 stream_bufs g_scr[MAX_SCR];
@@ -221,8 +221,10 @@ bool split_scratch(hipStream_t s, size_t bytes_o, size_t bytes_ml, float *& o, f
 // The library's own f16 staging copy for a prefill over a quantized cache without caller scratch: a buffer of at least
 // `bytes` bytes of (current device, s), or nullptr when there is none to be had now - over the limit, allocation failed, or
 // the stream is being captured and the buffer would have to be allocated or grown. Never an error: the caller then
-// converts inside the kernel, with the same result bits. Grown in steps (64 MiB granules, at least half as much again),
-// replaced buffers stay allocated until p1a_release() like every buffer a captured graph may hold.
+// converts inside the kernel, with the same result bits. Grown in steps (64 MiB granules, at least half as much again).
+// A replaced buffer is freed on the spot (hipFree waits for the work that still reads it) unless a call under stream
+// capture has been handed it - a captured graph holds its address - in which case it stays allocated until
+// p1a_release(): what the library keeps per (device, stream) is at most the limit, plus what graphs pin.
 void * stage_scratch(hipStream_t s, size_t bytes) {
     int dev = 0;
     if (!bytes || bytes > g_stage_limit || hipGetDevice(&dev) != hipSuccess) return nullptr;
@@ -234,10 +236,11 @@ void * stage_scratch(hipStream_t s, size_t bytes) {
         e = &g_scr[g_nscr++];
         e->dev = dev; e->s = s;
     }
-    if (bytes <= e->cap_stage) return e->stage;
     hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
-    if (s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone) return nullptr;
-    if (e->stage && g_nretired + 1 > MAX_RETIRED) return nullptr;
+    const bool capturing = s && hipStreamIsCapturing(s, &st) == hipSuccess && st != hipStreamCaptureStatusNone;
+    if (bytes <= e->cap_stage) { if (capturing) e->stage_captured = true; return e->stage; }
+    if (capturing) return nullptr;
+    if (e->stage && e->stage_captured && g_nretired + 1 > MAX_RETIRED) return nullptr;
     const size_t gran = (size_t) 64 << 20;
     size_t want = (bytes + gran - 1) / gran * gran;
     if (want < e->cap_stage + e->cap_stage / 2) want = e->cap_stage + e->cap_stage / 2;
@@ -245,8 +248,11 @@ void * stage_scratch(hipStream_t s, size_t bytes) {
     if (want < bytes) want = bytes;
     void * p = nullptr;
     if (hipMalloc(&p, want) != hipSuccess) { (void) hipGetLastError(); return nullptr; }
-    if (e->stage) g_retired[g_nretired++] = retired{dev, e->stage};
-    e->stage = p; e->cap_stage = want;
+    if (e->stage) {
+        if (e->stage_captured) g_retired[g_nretired++] = retired{dev, e->stage};
+        else (void) hipFree(e->stage);
+    }
+    e->stage = p; e->cap_stage = want; e->stage_captured = false;
     return p;
 }
 
