@@ -127,6 +127,9 @@ int p1a_attn_prep_mrope(const float *qg, const float *k, const float *v, const f
  * Without pos_rows all T rows belong to one sequence and share the KV read in groups of up to 4 rows.
  * The key partition does not depend on T, p0 or the batch composition: row t of any call is bitwise the T = 1 call
  * at pos(t) on that sequence, and a paged cache gives the bits of the contiguous one.
+ * Shapes: any D % 32 == 0 up to 512 and any Hq % Hkv == 0; the matrix-pipe kernels take D = 64 / 128 / 256 with Hq / Hkv <= 16
+ * and pages of >= 16 positions (f16 and the quantized types at D = 256 with 16-byte aligned bases and page strides, the
+ * quantized types at D = 64 / 128 with 4-byte aligned ones), everything else a slow generic kernel.
  * Replaces attn_decode (src/fast/attn.cuh:44, attn.cu:638-648), attn_decode_dev (attn.cuh:59-60, attn.cu:656-666),
  * attn_decode_rows (attn.cuh:64-65, attn.cu:650-654) and attn_decode2 (src/fast/attn_dec2.cuh:17-18); the gate
  * replaces the separate sigmoid_mul launch (src/kernels.cu:85-93).
@@ -220,10 +223,11 @@ int p1a_get_nsplit(int Hkv);
 void p1a_set_nsplit(int n);
 /* Bytes of split scratch one decode call of these arguments needs (accumulators rounded up to 256 bytes, then the (m, l)
  * pairs), and the bytes the library keeps per (device, stream) for a head shape - the larger of the two is what a first call
- * allocates. A cache the MFMA kernel cannot take (misaligned base or page stride, pages of fewer than 16 positions, quantized
- * types at D != 256) takes the generic kernel, which leaves more partials per row; both are covered. No GPU call is made
+ * allocates. A cache the MFMA kernel cannot take (misaligned base or page stride, pages of fewer than 16 positions, head
+ * sizes other than 64 / 128 / 256) takes the generic kernel, which leaves more partials per row; both are covered. No GPU call is made
  * (without a device the plan of a 256-CU part is returned). No counterpart in the reference, whose scratch size is a
- * compile-time constant (src/fast/attn_dec2.cu:452-464). */
+ * compile-time constant (src/fast/attn_dec2.cu:452-464). rows_per_seq as for p1a_attn_decode (T for a call without
+ * pos_rows). */
 size_t p1a_decode_scratch_bytes(const p1a_kv *c, int Hq, int T, int rows_per_seq);
 size_t p1a_decode_footprint_bytes(int Hq, int Hkv, int D);
 /* An identity of everything in this library that can change output BITS for a head shape on the current device: library

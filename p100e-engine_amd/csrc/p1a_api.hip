@@ -147,7 +147,7 @@ void decode_footprint(int Hq, int Hkv, int D, size_t & need_o, size_t & need_ml)
     const uint32_t types[3] = {P1A_KV_F16, P1A_KV_Q8_0, P1A_KV_Q4_0};
     // (a cache the MFMA kernel cannot take - a misaligned base, short pages - goes to the generic kernel, which leaves more
     // partials per row: both plans count, so that a warm-up also covers such caches)
-    for (uintptr_t base : {(uintptr_t) 16, (uintptr_t) 8})
+    for (uintptr_t base : {(uintptr_t) 16, (uintptr_t) 2})
         for (uint32_t ty : types)
             for (int rg = 1; rg <= 4; ++rg) {
                 size_t o, m;
