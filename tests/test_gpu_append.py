@@ -109,3 +109,41 @@ def test_fill_random_bytes(p1a, kv_type):
     out = torch.empty((2, Hq, D), device="cuda")
     p1a.attn_decode(dev(q), pool.dev_seq(0), out, 2, 698, Hq, 1 / 16, gate=dev(gate))
     check(out.cpu().numpy(), ref, f"decode over a filled cache, type {kv_type}")
+
+
+@pytest.mark.parametrize("kv_type", [O.KV_Q8_0, O.KV_Q4_0])
+def test_half_way_points_and_golden_blocks_in_a_long_call(p1a, kv_type):
+    """a call of a thousand rows: the reference quantizer's golden blocks - edge cases included - and blocks crafted so that
+    x / d lands exactly on half-way points (x.5 must round away from zero), just inside them, on the clamp (q4_0: code
+    16 -> 15) and on signed zeros, byte for byte the oracle's"""
+    gold = GOLD["x"]
+    n = gold.shape[0] // 8 * 8
+    g = I.rng(4242)
+    crafted = np.zeros((2048, 32), np.float32)
+    for b in range(crafted.shape[0]):
+        top = float(g.choice([127.0, 63.5, 254.0, 8.0, 1.0, 16.0, 0.5]))
+        sign = -1.0 if b % 3 == 0 else 1.0
+        crafted[b, 0] = sign * top                                  # the block maximum: d = top / 127 (q8_0), -+top / 8 (q4_0)
+        ks = g.integers(-126, 127, 31).astype(np.float32)
+        d8 = top / 127.0
+        half = (ks + np.where(ks >= 0, 0.5, -0.5)) * d8             # exact half-way points of the q8_0 grid where representable
+        near = np.nextafter(half.astype(np.float32), np.float32(0)) # ... and the float just inside them
+        crafted[b, 1:] = np.where(g.integers(0, 3, 31) == 0, near, half).astype(np.float32)
+        if b % 7 == 0:
+            crafted[b, 5:9] = [0.0, -0.0, top / 16.0, -top / 16.0]
+    x = np.concatenate([gold[:n], gold[:n], crafted.reshape(-1, 32)]).astype(np.float32)
+    nb = x.shape[0] // 8 * 8
+    rows = np.ascontiguousarray(x[:nb].reshape(nb // 8, 1, 256))
+    host = O.HostKV.contiguous(kv_type, nb // 8, 1, 256)
+    O.kv_append_rows(host, rows, rows[::-1].copy(), np.arange(nb // 8))
+    c = p1a.KVCache.contiguous(kv_type, nb // 8, 1, 256)
+    p1a.kv_append(c, dev(rows), dev(rows[::-1].copy()), 0, nb // 8)
+    torch.cuda.synchronize()
+    assert np.array_equal(c._keep[0].cpu().numpy(), host.k)
+    assert np.array_equal(c._keep[1].cpu().numpy(), host.v)
+    # and the golden bytes themselves
+    got = c._keep[0].cpu().numpy().reshape(nb // 8, -1)[:n // 8]
+    if kv_type == O.KV_Q8_0:
+        assert np.array_equal(got[:, 16:].copy().view(np.int8).reshape(n, 32), GOLD["q8_q"][:n])
+    else:
+        assert np.array_equal(got.reshape(n, 18), GOLD["q4_blk"][:n])
