@@ -235,7 +235,7 @@ size_t p1a_decode_footprint_bytes(int Hq, int Hkv, int D);
  * equal ids produce bit-identical attention outputs for equal inputs; the engine folds such switches into the numerics
  * hash of its session files (src/tp_model.cu:3697-3735). The prefill key-split plan is a function of (T, p0, Hq) and the
  * CU count, so it is covered. */
-#define P1A_NUMERICS_REV 3
+#define P1A_NUMERICS_REV 4
 uint64_t p1a_numerics_id(int Hq, int Hkv);
 /* Re-read the environment switch that is baked into captured graphs (P1A_DEC_SPLIT, the split-stream count); returns 1
  * when it differs from what was last read - the very first read included, as in the reference - (the caller must then drop
